@@ -10,6 +10,7 @@ from .registry import (
 from . import llama as _llama  # registers LlamaForCausalLM
 from . import buderax as _buderax  # registers Buderax
 from . import gisodra as _gisodra  # registers Gisodra
+from . import zudisun as _zudisun  # registers Zudisun
 
 __all__ = [
     "Architecture",

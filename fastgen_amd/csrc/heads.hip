@@ -32,6 +32,9 @@ struct PrepareArgs {
   int rot_q, rot_k;                  // whether the query heads turn, and the key heads
   float eps;
   const int* slots; void* k_pages; void* v_pages; int page_size, hd_c;  // hd_c: the cache's head size
+  int norm_plain;                    // a head with norm dims and no norm weight is divided by its root mean square
+  const int* positions; float q_temp_coef; int q_temp_every;  // queries times 1 + coef * ln(floor((p + 1) / every) + 1)
+  const void* v_first; int v_first_stride; float v_blend;     // values become (1 - v_blend) v + v_blend v_first[t, head, :]
 };
 
 // grid (T, ceil((n_q + n_kv) / HP_WAVES)); a wave a (token, head).  Lane l holds the pairs l, l + 64, ..
@@ -68,16 +71,26 @@ __global__ __launch_bounds__(HP_WAVES* FG_WAVE) void heads_prepare_kernel(const 
       if (d < norm_dims) ss += x[j][0] * x[j][0] + x[j][1] * x[j][1];
     }
   }
-  if (norm_w) {  // uniform
+  // a query's temperature grows with the logarithm of its position, in steps of `every` positions
+  const bool tempered = is_q && a.positions && a.q_temp_every > 0;  // uniform
+  const float temp = tempered ? 1.f + a.q_temp_coef * logf((float)((a.positions[t] + 1) / a.q_temp_every) + 1.f) : 1.f;
+  if (norm_w || (a.norm_plain && norm_dims > 0)) {  // uniform
     ss = wave_sum(ss);
     const float rstd = rsqrtf(ss / (float)norm_dims + a.eps);
 #pragma unroll
     for (int j = 0; j < HP_MAX_PAIRS; ++j) {
       const int d = 2 * (lane + FG_WAVE * j);
       if (d < norm_dims) {
-        x[j][0] = x[j][0] * rstd * norm_w[d];
-        x[j][1] = x[j][1] * rstd * norm_w[d + 1];
+        x[j][0] = x[j][0] * rstd * (norm_w ? norm_w[d] : 1.f);
+        x[j][1] = x[j][1] * rstd * (norm_w ? norm_w[d + 1] : 1.f);
       }
+    }
+  }
+  if (tempered) {
+#pragma unroll
+    for (int j = 0; j < HP_MAX_PAIRS; ++j) {
+      x[j][0] *= temp;
+      x[j][1] *= temp;
     }
   }
   if (a.table && (is_q ? a.rot_q : a.rot_k)) {  // uniform
@@ -125,6 +138,11 @@ __global__ __launch_bounds__(HP_WAVES* FG_WAVE) void heads_prepare_kernel(const 
           const int c = a.v_col + head * a.v_w + d;
           v0 = to_f<TS>(row[c]) + (a.bias ? a.bias[c] : 0.f);
           v1 = to_f<TS>(row[c + 1]) + (a.bias ? a.bias[c + 1] : 0.f);
+          if (a.v_first) {  // blended with the values that an earlier layer computed for this token
+            const TS* f = (const TS*)a.v_first + (size_t)t * a.v_first_stride + head * a.v_w + d;
+            v0 = (1.f - a.v_blend) * v0 + a.v_blend * to_f<TS>(f[0]);
+            v1 = (1.f - a.v_blend) * v1 + a.v_blend * to_f<TS>(f[1]);
+          }
         }
       }
       vp[lay.v_off(off, d)] = from_f<TA>(v0);

@@ -25,14 +25,27 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // wave in a fixed order), into LDS.  Few tokens (decode) get 16 waves a token and 2 experts a turn, so that
 // the router's rows are asked for by many waves at once; many tokens 4 waves and 4 experts a turn.  Then the `top` largest (ties: the lower expert) by a
 // wave-wide argmax repeated `top` times, and the softmax over them; every wave does this on the same LDS
-// values, the first one stores.  LDS: n_experts logits, then `top` chosen values.
+// values, the first one stores.  LDS: n_experts logits, then `top` chosen values, then n_experts scores.
+//
+// A second way of scoring (`sigmoid_scores`): an expert's score is sigmoid(logit); the choice goes by the
+// score plus `correction` (per expert, or null), inside the `keep_groups` best of `n_groups` groups of
+// neighbouring experts (a group's rank: the sum of its two largest choice scores; the experts of the other
+// groups cannot be chosen); the weights are the chosen experts' scores without the correction, divided by
+// their sum (+ 1e-20) and multiplied by `weight_scale`.
+struct RouteMode {
+  int sigmoid_scores;
+  const float* correction;
+  int n_groups, keep_groups;
+  float weight_scale;
+};
 template <class T, int WAVES, int EPW>
 __global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
     const T* __restrict__ x, int ldx, const float* __restrict__ wr, const float* __restrict__ bias,
-    int dim, int n_experts, int top, int* __restrict__ choice, float* __restrict__ weight) {
+    int dim, int n_experts, int top, int* __restrict__ choice, float* __restrict__ weight, const RouteMode mode) {
   extern __shared__ float lds[];
   float* z = lds;
   float* chosen = lds + n_experts;
+  float* score = chosen + top;
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const size_t t = blockIdx.x;
   const T* xr = x + t * ldx;
@@ -66,6 +79,41 @@ __global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
     }
   }
   __syncthreads();
+  if (mode.sigmoid_scores) {  // uniform
+    for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+      const float sc = 1.f / (1.f + expf(-z[e]));
+      score[e] = sc;
+      z[e] = sc + (mode.correction ? mode.correction[e] : 0.f);
+    }
+    __syncthreads();
+    if (mode.n_groups > 1 && mode.keep_groups < mode.n_groups) {  // uniform
+      // one wave ranks the groups (a lane a group, in turns) and strikes the experts of those that lose
+      float* rank = score + n_experts;  // n_groups values
+      const int per = n_experts / mode.n_groups;
+      if (wave == 0) {
+        for (int g = lane; g < mode.n_groups; g += FG_WAVE) {
+          float a = -INFINITY, b = -INFINITY;  // the two largest
+          for (int i = 0; i < per; ++i) {
+            const float v = z[g * per + i];
+            if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+          }
+          rank[g] = per > 1 ? a + b : a;
+        }
+      }
+      __syncthreads();
+      if (wave == 0) {
+        for (int g = lane; g < mode.n_groups; g += FG_WAVE) {
+          // a group stays if fewer than keep_groups groups rank before it (ties: the lower group first)
+          int before = 0;
+          const float mine = rank[g];
+          for (int o = 0; o < mode.n_groups; ++o) before += (rank[o] > mine || (rank[o] == mine && o < g)) ? 1 : 0;
+          if (before >= mode.keep_groups)
+            for (int i = 0; i < per; ++i) z[g * per + i] = -INFINITY;
+        }
+      }
+      __syncthreads();
+    }
+  }
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
     int at = 0x7fffffff;
@@ -83,12 +131,16 @@ __global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
     if (threadIdx.x == 0) {
       at = min(at, n_experts - 1);  // (only if every logit is NaN)
       z[at] = -INFINITY;
-      chosen[j] = best;
+      chosen[j] = mode.sigmoid_scores ? score[at] : best;
       choice[t * top + j] = at;
     }
     __syncthreads();
   }
-  if (threadIdx.x == 0) {
+  if (threadIdx.x == 0 && mode.sigmoid_scores) {
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) sum += chosen[j];
+    for (int j = 0; j < top; ++j) weight[t * top + j] = chosen[j] / (sum + 1e-20f) * mode.weight_scale;
+  } else if (threadIdx.x == 0) {
     const float m = chosen[0];  // the largest
     float sum = 0.f;
     for (int j = 0; j < top; ++j) sum += expf(chosen[j] - m);
@@ -96,15 +148,21 @@ __global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
   }
 }
 
-extern "C" int fg_moe_route(const void* x, int ldx, int dtype, const float* wr, const float* bias, int n_tokens, int dim,
-                            int n_experts, int top, int* choice, float* weight, hipStream_t stream) {
+extern "C" int fg_moe_route_mode(const void* x, int ldx, int dtype, const float* wr, const float* bias, int n_tokens,
+                                 int dim, int n_experts, int top, int* choice, float* weight, int sigmoid_scores,
+                                 const float* correction, int n_groups, int keep_groups, float weight_scale,
+                                 hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
   if (dim <= 0 || ldx < dim || n_experts <= 0 || top < 1 || top > n_experts) return FG_ERR_ARG;
-  const size_t lds = (size_t)(n_experts + top) * sizeof(float);
+  if (n_groups < 1 || n_experts % n_groups || keep_groups < 1 || keep_groups > n_groups ||
+      top > keep_groups * (n_experts / n_groups) || (!sigmoid_scores && (correction || n_groups > 1)))
+    return FG_ERR_ARG;
+  const RouteMode mode = {sigmoid_scores, correction, n_groups, keep_groups, weight_scale};
+  const size_t lds = (size_t)(2 * n_experts + top + n_groups) * sizeof(float);
   if (lds > 60000) return FG_ERR_ARG;
 #define GO(T, WAVES, EPW)                                                                                        \
   moe_route_kernel<T, WAVES, EPW><<<n_tokens, 64 * WAVES, lds, stream>>>((const T*)x, ldx, wr, bias, dim, n_experts, \
-                                                                         top, choice, weight)
+                                                                         top, choice, weight, mode)
   const bool few = n_tokens <= 64;
   if (dtype == FG_F32) {
     if (few) GO(float, 16, 2); else GO(float, 4, 4);
@@ -115,6 +173,12 @@ extern "C" int fg_moe_route(const void* x, int ldx, int dtype, const float* wr, 
   }
 #undef GO
   return fg_launch_status();
+}
+
+extern "C" int fg_moe_route(const void* x, int ldx, int dtype, const float* wr, const float* bias, int n_tokens, int dim,
+                            int n_experts, int top, int* choice, float* weight, hipStream_t stream) {
+  return fg_moe_route_mode(x, ldx, dtype, wr, bias, n_tokens, dim, n_experts, top, choice, weight, 0, nullptr, 1, 1, 1.f,
+                           stream);
 }
 
 // -------------------------------------------------------------------- sort

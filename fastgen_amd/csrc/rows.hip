@@ -402,18 +402,22 @@ extern "C" int fg_silu_mul(const void* gu, void* out, int n_rows, int hidden, in
 //   h += d * rsqrt(mean(d^2) + eps_p) * wp ;  out = h * rsqrt(mean(h^2) + eps) * w
 // all in fp32 with one rounding at the store of `out`.  With `rows` only the gathered rows are
 // computed and h is left as it was.  A thread keeps its elements i = tid, tid + 256, .. in registers.
+// `dbias` (fp32 per column, or null) is added to d before its norm (a projection's bias).  Without `w` but
+// with `out` the stream's row itself is stored, rounded to the activation dtype: what a sublayer reads
+// that takes the stream un-normed.  Without delta and parts nothing is added.
 #define POST_MAX_PER_THREAD 64  // rows of up to 16,384 elements
 template <class TA, class TW, int NIT>
 __global__ __launch_bounds__(ROWS_THREADS) void post_add_rmsnorm_kernel(
     float* __restrict__ h, const TA* __restrict__ delta, const float* __restrict__ parts, int n_parts,
     size_t part_stride, const TW* __restrict__ wp, float eps_p, const TW* __restrict__ w, TA* __restrict__ out,
-    const int* __restrict__ rows, int dim, float eps) {
+    const int* __restrict__ rows, int dim, float eps, const float* __restrict__ dbias) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
   float* hrow = h + src * dim;
   float d[NIT];
   float ss = 0.f;
+  const bool adds = delta || parts;  // uniform
 #pragma unroll
   for (int j = 0; j < NIT; ++j) {
     const int i = threadIdx.x + j * ROWS_THREADS;
@@ -422,6 +426,7 @@ __global__ __launch_bounds__(ROWS_THREADS) void post_add_rmsnorm_kernel(
     if (delta) v = to_f<TA>(delta[src * dim + i]);
     if (parts)
       for (int p = 0; p < n_parts; ++p) v += parts[p * part_stride + src * dim + i];
+    if (dbias && adds) v += dbias[i];
     d[j] = v;
     ss += v * v;
   }
@@ -432,35 +437,38 @@ __global__ __launch_bounds__(ROWS_THREADS) void post_add_rmsnorm_kernel(
   for (int j = 0; j < NIT; ++j) {
     const int i = threadIdx.x + j * ROWS_THREADS;
     if (i >= dim) continue;
-    const float v = hrow[i] + d[j] * rstd_p * to_f<TW>(wp[i]);
-    if (!rows) hrow[i] = v;
+    const float v = adds ? hrow[i] + d[j] * rstd_p * to_f<TW>(wp[i]) : hrow[i];
+    if (!rows && adds) hrow[i] = v;
     d[j] = v;
     s2 += v * v;
   }
-  if (!w) return;  // uniform
-  s2 = block_sum(s2, red);
-  const float rstd = rsqrtf(s2 / (float)dim + eps);
+  if (!out) return;  // uniform
+  float rstd = 1.f;
+  if (w) {  // uniform
+    s2 = block_sum(s2, red);
+    rstd = rsqrtf(s2 / (float)dim + eps);
+  }
   TA* orow = out + (size_t)r * dim;
 #pragma unroll
   for (int j = 0; j < NIT; ++j) {
     const int i = threadIdx.x + j * ROWS_THREADS;
     if (i >= dim) continue;
-    orow[i] = from_f<TA>(d[j] * rstd * to_f<TW>(w[i]));
+    orow[i] = from_f<TA>(w ? d[j] * rstd * to_f<TW>(w[i]) : d[j]);
   }
 }
 
 extern "C" int fg_post_add_rmsnorm(float* h, const void* delta, const float* parts, int n_parts,
                                    long long part_stride, const void* wp, float eps_p, const void* w, void* out,
                                    const int* rows, int n_rows, int dim, float eps, int act_dtype, int w_dtype,
-                                   hipStream_t stream) {
+                                   const float* dbias, hipStream_t stream) {
   if (n_rows <= 0) return FG_OK;
-  if (dim <= 0 || dim > POST_MAX_PER_THREAD * ROWS_THREADS || (parts && n_parts < 1) || !wp || (w && !out) ||
-      (!delta && !parts))
+  if (dim <= 0 || dim > POST_MAX_PER_THREAD * ROWS_THREADS || (parts && n_parts < 1) || (w && !out) ||
+      ((delta || parts) && !wp) || (!delta && !parts && !out))
     return FG_ERR_ARG;
 #define GO(TA, TW, NIT)                                                                                       \
   post_add_rmsnorm_kernel<TA, TW, NIT><<<n_rows, ROWS_THREADS, 0, stream>>>(                                  \
       h, (const TA*)delta, parts, n_parts, (size_t)part_stride, (const TW*)wp, eps_p, (const TW*)w, (TA*)out, \
-      rows, dim, eps)
+      rows, dim, eps, dbias)
 #define LAUNCH(TA, TW)                                 \
   do {                                                 \
     if (dim <= 4 * ROWS_THREADS) GO(TA, TW, 4);        \
@@ -512,6 +520,61 @@ extern "C" int fg_gelu_mul(const void* gu, void* out, int n_rows, int hidden, in
     else if (act_dtype == FG_BF16)
       gelu_mul_vec_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>((const bf16_t*)gu + (size_t)r0 * 2 * hidden,
                                                                      (bf16_t*)out + (size_t)r0 * hidden, hidden);
+    else
+      return FG_ERR_ARG;
+  }
+  return fg_launch_status();
+}
+
+// ------------------------------------------- act(g + b) * (u + b), any source dtype
+// The general form of the two kernels above: the rows may be fp32 (a product's un-rounded result) while
+// the result has the activation dtype, a bias per column of gu (fp32, in gu's interleaved order) is added
+// first, and the activation is SiLU (0), the tanh form of GELU (1) or ReLU (2).  All of it in fp32.
+template <class TS, class TA>
+__global__ __launch_bounds__(ROWS_THREADS) void gated_mul_kernel(
+    const TS* __restrict__ gu, const float* __restrict__ bias, TA* __restrict__ out, int hidden, int act) {
+  const TS* row = gu + (size_t)blockIdx.y * 2 * hidden;
+  TA* o = out + (size_t)blockIdx.y * hidden;
+  const int e = (blockIdx.x * ROWS_THREADS + threadIdx.x) * 8;
+  if (e < hidden) {
+    float gv[8], uv[8], r[8];
+    load8<TS>(row + 2 * e, gv);
+    load8<TS>(row + 2 * e + 8, uv);
+    if (bias) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        gv[i] += bias[2 * e + i];
+        uv[i] += bias[2 * e + 8 + i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float g = gv[i];
+      float a;
+      if (act == 0) a = g / (1.f + expf(-g));
+      else if (act == 1) a = 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+      else a = fmaxf(g, 0.f);
+      r[i] = a * uv[i];
+    }
+    store8<TA>(o + e, r);
+  }
+}
+
+extern "C" int fg_gated_mul(const void* gu, const float* bias, void* out, int n_rows, int hidden, int act,
+                            int src_dtype, int act_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (hidden <= 0 || hidden % 8 || n_rows > 65535 * 32 || act < 0 || act > 2) return FG_ERR_ARG;
+  for (int r0 = 0; r0 < n_rows; r0 += 65535) {
+    const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
+    const int per_block = ROWS_THREADS * 8;
+    dim3 grid((hidden + per_block - 1) / per_block, nr);
+    const size_t so = (size_t)r0 * 2 * hidden, oo = (size_t)r0 * hidden;
+    if (src_dtype == FG_F32 && act_dtype == FG_F32)
+      gated_mul_kernel<float, float><<<grid, ROWS_THREADS, 0, stream>>>((const float*)gu + so, bias, (float*)out + oo, hidden, act);
+    else if (src_dtype == FG_F32 && act_dtype == FG_BF16)
+      gated_mul_kernel<float, bf16_t><<<grid, ROWS_THREADS, 0, stream>>>((const float*)gu + so, bias, (bf16_t*)out + oo, hidden, act);
+    else if (src_dtype == FG_BF16 && act_dtype == FG_BF16)
+      gated_mul_kernel<bf16_t, bf16_t><<<grid, ROWS_THREADS, 0, stream>>>((const bf16_t*)gu + so, bias, (bf16_t*)out + oo, hidden, act);
     else
       return FG_ERR_ARG;
   }

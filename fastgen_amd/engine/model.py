@@ -183,7 +183,7 @@ class Model:
             block = blocks[entry.layer]
             if entry.inject is not None:
                 if isinstance(pending, PostNormed):  # a sublayer's output that is normed before it is added
-                    post_add_rmsnorm(h, pending.rows, pending.weight, pending.eps, None, 0.0, None)
+                    post_add_rmsnorm(h, pending.rows, pending.weight, pending.eps, None, 0.0, None, delta_bias=pending.bias)
                     pending = None
                 injections[entry.inject[0]].forward(h, None if isinstance(pending, ScaledRows) else pending,
                                                     embedded, entry.inject[1])

@@ -47,6 +47,8 @@ LIBRARIES: Dict[str, str] = {
     "moe": "moe.hip",
     "heads": "heads.hip",
     "recurrence": "recurrence.hip",
+    "selective_scan": "selective_scan.hip",
+    "sigmoid_attention": "sigmoid_attention.hip",
 }
 
 # libraries compiled once per value of a macro: name -> (source, macro, values that build_all compiles,

@@ -260,35 +260,46 @@ class PostNormed:
     rows: torch.Tensor
     weight: torch.Tensor
     eps: float
+    bias: Optional[torch.Tensor] = None  # fp32 [dim]: added to the rows before their norm (a projection's bias)
 
 
-def post_add_rmsnorm(h: torch.Tensor, delta: torch.Tensor, post_weight: torch.Tensor, post_eps: float,
-                     weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
-                     rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-    """``h += rmsnorm(delta) * post_weight`` on the fp32 stream ``h [T, dim]`` and, with ``weight``,
+def post_add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], post_weight: Optional[torch.Tensor],
+                     post_eps: float, weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
+                     rows: Optional[torch.Tensor] = None, delta_bias: Optional[torch.Tensor] = None
+                     ) -> Optional[torch.Tensor]:
+    """``h += rmsnorm(delta + delta_bias) * post_weight`` on the fp32 stream ``h [T, dim]`` and, with ``weight``,
     ``out = rmsnorm(h) * weight``: the norm behind a sublayer, the addition and the norm before the next
-    one in one pass, all in fp32.  ``delta`` as :func:`add_rmsnorm` takes it.  With ``rows`` only those
-    rows are computed, into consecutive rows of ``out``, and ``h`` is left as it was."""
-    _gpu(h, delta, post_weight, weight, out, rows)
+    one in one pass, all in fp32.  ``delta`` as :func:`add_rmsnorm` takes it; None: nothing is added.  With
+    ``out`` but without ``weight`` the stream's rows themselves are stored, rounded to ``out``'s dtype (what a
+    sublayer reads that takes the stream un-normed).  With ``rows`` only those rows are computed, into
+    consecutive rows of ``out``, and ``h`` is left as it was."""
+    _gpu(h, delta, post_weight, weight, out, rows, delta_bias)
     _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "h must be contiguous float32 [T, dim]")
     T, dim = h.shape
     n_rows = T if rows is None else rows.numel()
     if rows is not None:
         _i32(rows, "rows")
-    _need(post_weight.shape == (dim,) and post_weight.is_contiguous(), "post_weight must be [dim]")
+    _need(delta is None or post_weight is not None, "rows that are added are normed: post_weight is missing")
+    _need(delta is not None or out is not None, "nothing to add and nothing to store")
+    if post_weight is not None:
+        _need(post_weight.shape == (dim,) and post_weight.is_contiguous(), "post_weight must be [dim]")
     if weight is not None:
-        _need(weight.shape == (dim,) and weight.is_contiguous() and weight.dtype == post_weight.dtype,
-              "weight must be [dim], of post_weight's dtype")
-        _need(out is not None and out.is_contiguous() and out.shape == (n_rows, dim), "out must be contiguous [rows, dim]")
+        _need(weight.shape == (dim,) and weight.is_contiguous()
+              and (post_weight is None or weight.dtype == post_weight.dtype), "weight must be [dim], of post_weight's dtype")
+    if out is not None:
+        _need(out.is_contiguous() and out.shape == (n_rows, dim), "out must be contiguous [rows, dim]")
     else:
-        _need(rows is None, "a gathered call computes the norm that follows")
+        _need(weight is None and rows is None, "a norm or a gathered call needs out")
+    _f32_vec(delta_bias, dim, "delta_bias")
     act = out.dtype if out is not None else (delta.dtype if delta.dim() == 2 else torch.float32)
     d_ptr, d_code, parts, n_parts, part_stride = _delta_args(h, delta, "post_add_rmsnorm")
-    if delta.dim() == 2:
+    if delta is not None and delta.dim() == 2:
         _need(delta.dtype == act, "delta must have out's dtype")
+    w_any = post_weight if post_weight is not None else weight
     st = _lib.load("rows").fg_post_add_rmsnorm(
         _ptr(h), d_ptr, parts, n_parts, part_stride, _ptr(post_weight), ctypes.c_float(post_eps), _ptr(weight),
-        _ptr(out), _ptr(rows), n_rows, dim, ctypes.c_float(eps), _DTYPE_CODE[act], _code(post_weight), _stream(h))
+        _ptr(out), _ptr(rows), n_rows, dim, ctypes.c_float(eps), _DTYPE_CODE[act],
+        _code(w_any) if w_any is not None else F32, _ptr(delta_bias), _stream(h))
     _check(st, "post_add_rmsnorm")
     return out
 
@@ -991,11 +1002,19 @@ def logprob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
 MOE_TILE_ROWS = (16, 32, 64, 128, 256)  # rows of one expert that a tile of the matrix-core kernels holds (from 128: through LDS)
 
 
-def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int,
+              sigmoid_scores: bool = False, correction: Optional[torch.Tensor] = None, n_groups: int = 1,
+              keep_groups: int = 1, weight_scale: float = 1.0):
     """Per row of ``x [T, dim]``: fp32 logits ``x router^T + bias`` (``router`` fp32 ``[E, dim]``), the
     ``top`` largest (ties: the lower expert), and the softmax over those.  Returns int32 ``[T, top]``
-    experts and fp32 ``[T, top]`` weights, the largest logit first."""
-    _gpu(x, router, bias)
+    experts and fp32 ``[T, top]`` weights, the largest logit first.
+
+    With ``sigmoid_scores`` an expert's score is ``sigmoid(logit)``; the choice goes by the score plus
+    ``correction`` (fp32 ``[E]`` or None) among the experts of the ``keep_groups`` best of ``n_groups`` equal
+    groups of neighbours (a group ranks by the sum of its two largest choice scores; ties: the lower group);
+    the weights are the chosen experts' scores, without the correction, divided by their sum (+ 1e-20)
+    and multiplied by ``weight_scale``."""
+    _gpu(x, router, bias, correction)
     _need(x.dim() == 2 and x.stride(1) == 1 and x.data_ptr() % 16 == 0, "x must be [T, dim] with unit column stride")
     T, dim = x.shape
     E = router.shape[0]
@@ -1006,8 +1025,13 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     _need(1 <= top <= E, f"top={top} must be between 1 and the {E} experts")
     choice = torch.empty((T, top), dtype=torch.int32, device=x.device)
     weight = torch.empty((T, top), dtype=torch.float32, device=x.device)
-    st = _lib.load("moe").fg_moe_route(_ptr(x), x.stride(0), _code(x), _ptr(router), _ptr(bias), T, dim, E, top,
-                                       _ptr(choice), _ptr(weight), _stream(x))
+    _f32_vec(correction, E, "correction")
+    _need(sigmoid_scores or (correction is None and n_groups == 1), "correction and groups go with sigmoid scores")
+    _need(n_groups >= 1 and E % n_groups == 0 and 1 <= keep_groups <= n_groups and top <= keep_groups * (E // n_groups),
+          f"{n_groups} groups of which {keep_groups} stay do not fit {E} experts and top={top}")
+    st = _lib.load("moe").fg_moe_route_mode(_ptr(x), x.stride(0), _code(x), _ptr(router), _ptr(bias), T, dim, E, top,
+                                            _ptr(choice), _ptr(weight), int(bool(sigmoid_scores)), _ptr(correction),
+                                            int(n_groups), int(keep_groups), ctypes.c_float(weight_scale), _stream(x))
     _check(st, "moe_route")
     return choice, weight
 
@@ -1117,7 +1141,9 @@ class _PrepareArgs(ctypes.Structure):
                 ("v_w", ctypes.c_int), ("table", ctypes.c_void_p), ("rot_start", ctypes.c_int),
                 ("rotary_dim", ctypes.c_int), ("rot_q", ctypes.c_int), ("rot_k", ctypes.c_int), ("eps", ctypes.c_float), ("slots", ctypes.c_void_p),
                 ("k_pages", ctypes.c_void_p), ("v_pages", ctypes.c_void_p), ("page_size", ctypes.c_int),
-                ("hd_c", ctypes.c_int)]
+                ("hd_c", ctypes.c_int), ("norm_plain", ctypes.c_int), ("positions", ctypes.c_void_p),
+                ("q_temp_coef", ctypes.c_float), ("q_temp_every", ctypes.c_int), ("v_first", ctypes.c_void_p),
+                ("v_first_stride", ctypes.c_int), ("v_blend", ctypes.c_float)]
 
 
 def _f32_vec(t: Optional[torch.Tensor], n: int, name: str) -> None:
@@ -1132,7 +1158,9 @@ def heads_prepare(src: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
                   k_norm_dims: int = 0, v_col: int = -1, v_width: int = 0,
                   table: Optional[torch.Tensor] = None, rot_start: int = 0, rotary_dim: int = 0,
                   rotate_q: bool = True, rotate_k: bool = True, slots: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
-                  v_pages: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                  v_pages: Optional[torch.Tensor] = None, norm_plain: bool = False,
+                  positions: Optional[torch.Tensor] = None, q_temp_coef: float = 0.0, q_temp_every: int = 0,
+                  v_first: Optional[torch.Tensor] = None, v_blend: float = 0.0) -> Optional[torch.Tensor]:
     """What lies between a product's rows ``src [T, width]`` (fp32, or the activation dtype) and an attention.
 
     Per token and head: add ``bias`` (fp32, per column of ``src``); RMS-norm the head's first ``*_norm_dims``
@@ -1143,8 +1171,13 @@ def heads_prepare(src: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
     The ``n_kv`` key heads (``k_width`` wide, from ``k_col``) go to ``slots`` of ``k_pages
     [n_pages, n_kv, P, hd]`` padded with zeros to ``hd``; the values (``v_width`` wide) to ``v_pages
     [n_pages, n_kv, hd, P]`` likewise: columns of their own from ``v_col``, with their bias, or, with
-    ``v_col < 0``, the first ``v_width`` elements of the processed key.  A negative slot writes nothing."""
-    _gpu(src, bias, q_norm, q_out, k_norm, table, slots, k_pages, v_pages)
+    ``v_col < 0``, the first ``v_width`` elements of the processed key.  A negative slot writes nothing.
+
+    ``norm_plain``: heads with norm dimensions but no norm weight are divided by their root mean square.
+    ``positions`` with ``q_temp_every > 0``: after its norm a query at position ``p`` is multiplied by
+    ``1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)``.  ``v_first [T, n_kv * v_width]`` (of ``src``'s
+    dtype, unit column stride): the values become ``(1 - v_blend) v + v_blend v_first`` before they are stored."""
+    _gpu(src, bias, q_norm, q_out, k_norm, table, slots, k_pages, v_pages, positions, v_first)
     _need(src.dim() == 2 and src.stride(1) == 1, "src must be [T, width] with unit column stride")
     T, width = src.shape
     a = _PrepareArgs()
@@ -1195,6 +1228,15 @@ def heads_prepare(src: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
         a.table, a.rot_start, a.rotary_dim = table.data_ptr(), rot_start, rotary_dim
         a.rot_q, a.rot_k = int(bool(rotate_q)), int(bool(rotate_k))
     _need(src.dtype == torch.float32 or src.dtype == act, "src must be float32 or of the cache's dtype")
+    a.norm_plain = int(bool(norm_plain))
+    if positions is not None and q_temp_every > 0:
+        _i32(positions, "positions", T)
+        a.positions, a.q_temp_coef, a.q_temp_every = positions.data_ptr(), float(q_temp_coef), int(q_temp_every)
+    if v_first is not None:
+        _need(n_kv > 0 and v_col >= 0, "blended values need values of their own to blend")
+        _need(v_first.dtype == src.dtype and v_first.dim() == 2 and v_first.stride(1) == 1 and v_first.shape[0] == T
+              and v_first.shape[1] >= n_kv * v_width, "v_first must be [T, >= n_kv * v_width] of src's dtype")
+        a.v_first, a.v_first_stride, a.v_blend = v_first.data_ptr(), v_first.stride(0), float(v_blend)
     st = _lib.load("heads").fg_heads_prepare(ctypes.byref(a), T, _code(src), _DTYPE_CODE[act], _stream(src))
     _check(st, "heads_prepare")
     return q_out
@@ -1336,4 +1378,209 @@ def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.T
                                      H, d, e, _stream(qkv)), "decay_chunk_states")
     a.write_out, a.write_state = 1, 0  # every chunk from the state it starts from
     _check(lib.fg_decay_scan(ctypes.byref(a), n_chunks, _code(qkv), _stream(qkv)), "decay_scan (chunks' outputs)")
+    return out
+
+
+# ----------------------------------------------------- gated activation, general
+_ACT_CODE = {"silu": 0, "gelu_tanh": 1, "relu": 2}
+
+
+def gated_mul(gate_up: torch.Tensor, bias: Optional[torch.Tensor], activation: str, out_dtype: torch.dtype,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``act(gate + b) * (up + b)`` for ``gate_up [T, 2 * hidden]`` as :func:`interleave_gate_up` orders it (fp32, or
+    ``out_dtype``), ``bias`` fp32 ``[2 * hidden]`` in the same order (or None), ``activation`` one of ``silu``,
+    ``gelu_tanh``, ``relu``.  All of it in fp32, one rounding to ``out_dtype``."""
+    _gpu(gate_up, bias, out)
+    _need(activation in _ACT_CODE, f"activation {activation!r} is not supported ({sorted(_ACT_CODE)})")
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 16 == 0,
+          "gate_up must be contiguous [T, 2 * hidden], hidden a multiple of 8")
+    T, hidden = gate_up.shape[0], gate_up.shape[1] // 2
+    _need(gate_up.dtype == torch.float32 or gate_up.dtype == out_dtype, "gate_up must be float32 or of the result's dtype")
+    _f32_vec(bias, 2 * hidden, "bias")
+    if out is None:
+        out = torch.empty((T, hidden), dtype=out_dtype, device=gate_up.device)
+    _need(out.shape == (T, hidden) and out.is_contiguous() and out.dtype == out_dtype, "out must be contiguous [T, hidden]")
+    st = _lib.load("rows").fg_gated_mul(_ptr(gate_up), _ptr(bias), _ptr(out), T, hidden, _ACT_CODE[activation],
+                                        _code(gate_up), _code(out), _stream(out))
+    _check(st, "gated_mul")
+    return out
+
+
+# ------------------------------------------------- selective state-space recurrence
+class _SelectiveArgs(ctypes.Structure):
+    _fields_ = [("u", ctypes.c_void_p), ("ldu", ctypes.c_int), ("dt", ctypes.c_void_p), ("lddt", ctypes.c_int),
+                ("dt_bias", ctypes.c_void_p), ("A", ctypes.c_void_p), ("bc", ctypes.c_void_p), ("ldbc", ctypes.c_int),
+                ("b_col", ctypes.c_int), ("c_col", ctypes.c_int), ("D", ctypes.c_void_p), ("z", ctypes.c_void_p),
+                ("ldz", ctypes.c_int), ("x_raw", ctypes.c_void_p), ("ldx", ctypes.c_int), ("state", ctypes.c_void_p),
+                ("row_len", ctypes.c_int), ("slot_ids", ctypes.c_void_p), ("q_start", ctypes.c_void_p),
+                ("out", ctypes.c_void_p), ("ldo", ctypes.c_int), ("C", ctypes.c_int), ("N", ctypes.c_int),
+                ("K", ctypes.c_int), ("LP", ctypes.c_int)]
+
+
+def _rows_of_width(t: torch.Tensor, T: int, width: int, name: str) -> None:
+    _need(t.dim() == 2 and t.stride(1) == 1 and t.shape[0] == T and t.shape[1] >= width,
+          f"{name} must be [T, >= {width}] with unit column stride")
+
+
+def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, tail_off: int,
+                slot_ids: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor, out: torch.Tensor,
+                activation: Optional[str] = None) -> torch.Tensor:
+    """A short causal convolution per channel over each sequence's tokens: ``out[t, c] = act(bias[c] + sum_j
+    taps[c, j] x[t - (K - 1) + j, c])``, the last tap on the token itself.  ``x [T, >= C]``; ``taps`` fp32
+    ``[C, K]``; tokens before this step's first are the last ``K - 1`` inputs of earlier steps, which
+    ``state`` fp32 ``[n_slots, C, row_len]`` holds from column ``tail_off`` on at row ``slot_ids[seq]`` (zeros for
+    a new request).  The state is read only (:func:`selective_scan` moves it on).  ``activation``: None or ``silu``."""
+    _gpu(x, taps, bias, state, slot_ids, seq_of_token, q_start, out)
+    C, K = taps.shape
+    T = x.shape[0]
+    _need(taps.dtype == torch.float32 and taps.is_contiguous(), "taps must be contiguous float32 [C, K]")
+    _f32_vec(bias, C, "bias")
+    _rows_of_width(x, T, C, "x")
+    _rows_of_width(out, T, C, "out")
+    _need(state.dtype == torch.float32 and state.dim() == 3 and state.is_contiguous() and state.shape[1] == C
+          and 0 <= tail_off and tail_off + K - 1 <= state.shape[2], "state must be contiguous float32 [n_slots, C, >= tail_off + K - 1]")
+    _need(activation in (None, "silu"), "activation must be None or 'silu'")
+    _i32(seq_of_token, "seq_of_token", T)
+    _i32(slot_ids, "slot_ids")
+    _i32(q_start, "q_start")
+    st = _lib.load("selective_scan").fg_causal_conv(
+        _ptr(x), x.stride(0), _ptr(taps), _ptr(bias), _ptr(state), state.shape[2], int(tail_off), _ptr(slot_ids),
+        _ptr(seq_of_token), _ptr(q_start), _ptr(out), out.stride(0), T, C, K, 1 if activation == "silu" else 0,
+        _code(x), _code(out), _stream(out))
+    _check(st, "causal_conv")
+    return out
+
+
+def selective_scan(u: torch.Tensor, dt: torch.Tensor, dt_bias: Optional[torch.Tensor], A: torch.Tensor, bc: torch.Tensor,
+                   b_col: int, c_col: int, D: Optional[torch.Tensor], z: Optional[torch.Tensor],
+                   x_raw: Optional[torch.Tensor], taps: int, state: torch.Tensor, slot_ids: torch.Tensor,
+                   q_start: torch.Tensor, n_seqs: int, out: torch.Tensor) -> torch.Tensor:
+    """The selective recurrence, token by token for every sequence of the step, in fp32:
+    ``d = softplus(dt[t, c] + dt_bias[c])``; ``S[c, n] <- exp(d A[c, n]) S[c, n] + d u[t, c] B[t, n]``;
+    ``out[t, c] = (sum_n S[c, n] C[t, n] + D[c] u[t, c]) * silu(z[t, c])``.
+
+    ``u [T, >= C]`` and ``out`` have the activation dtype; ``dt [T, >= C]`` is fp32 or of the activation dtype; ``A``
+    fp32 ``[C, N]``; ``B[t, n] = bc[t, b_col + n]``, ``C[t, n] = bc[t, c_col + n]``; ``state`` fp32 ``[n_slots, C,
+    row_len]`` holds ``S`` in its first ``N`` columns and, behind them, the last ``taps - 1`` rows of ``x_raw`` (the
+    input of the convolution that made ``u``), which this call moves on by the step's tokens.  Sequence ``b`` has
+    the tokens ``q_start[b] .. q_start[b+1]-1`` and the state row ``slot_ids[b]``."""
+    _gpu(u, dt, dt_bias, A, bc, D, z, x_raw, state, slot_ids, q_start, out)
+    C, N = A.shape
+    T = u.shape[0]
+    act = out.dtype
+    _need(A.dtype == torch.float32 and A.is_contiguous(), "A must be contiguous float32 [C, N]")
+    _rows_of_width(u, T, C, "u")
+    _rows_of_width(dt, T, C, "dt")
+    _rows_of_width(out, T, C, "out")
+    _need(u.dtype == act and bc.dtype == act and dt.dtype in (torch.float32, act), "u, bc and out share a dtype; dt is float32 or of it")
+    _need(min(b_col, c_col) >= 0, "B and C must lie inside the rows of bc")
+    _rows_of_width(bc, T, max(b_col, c_col) + N, "bc")
+    _f32_vec(dt_bias, C, "dt_bias")
+    _f32_vec(D, C, "D")
+    a = _SelectiveArgs()
+    if z is not None:
+        _rows_of_width(z, T, C, "z")
+        _need(z.dtype == act, "z must have out's dtype")
+        a.z, a.ldz = z.data_ptr(), z.stride(0)
+    _need(taps >= 1 and (taps == 1 or x_raw is not None), "the convolution's input is needed to move its tail on")
+    if taps > 1:
+        _rows_of_width(x_raw, T, C, "x_raw")
+        _need(x_raw.dtype == act, "x_raw must have out's dtype")
+        a.x_raw, a.ldx = x_raw.data_ptr(), x_raw.stride(0)
+    _need(state.dtype == torch.float32 and state.dim() == 3 and state.is_contiguous() and state.shape[1] == C
+          and state.shape[2] >= N + taps - 1, "state must be contiguous float32 [n_slots, C, >= N + taps - 1]")
+    _i32(slot_ids, "slot_ids", n_seqs)
+    _i32(q_start, "q_start", n_seqs + 1)
+    spl = 4 if N <= 256 else 8 if N <= 512 else 16
+    lanes = 1
+    while lanes * spl < N:
+        lanes *= 2
+    _need(lanes <= 64, "at most 1024 states a channel")
+    a.u, a.ldu, a.dt, a.lddt = u.data_ptr(), u.stride(0), dt.data_ptr(), dt.stride(0)
+    a.dt_bias, a.A, a.D = (dt_bias.data_ptr() if dt_bias is not None else None), A.data_ptr(), (D.data_ptr() if D is not None else None)
+    a.bc, a.ldbc, a.b_col, a.c_col = bc.data_ptr(), bc.stride(0), int(b_col), int(c_col)
+    a.state, a.row_len, a.slot_ids, a.q_start = state.data_ptr(), state.shape[2], slot_ids.data_ptr(), q_start.data_ptr()
+    a.out, a.ldo, a.C, a.N, a.K, a.LP = out.data_ptr(), out.stride(0), C, N, int(taps), lanes
+    st = _lib.load("selective_scan").fg_selective_scan(ctypes.byref(a), int(n_seqs), _code(dt), _code(out), _stream(out))
+    _check(st, "selective_scan")
+    return out
+
+
+# ----------------------------------------------------------- sigmoid attention
+class _SigmoidAttentionArgs(ctypes.Structure):
+    _fields_ = [("q", ctypes.c_void_p), ("q_stride", ctypes.c_int), ("q_hs", ctypes.c_int), ("k_pages", ctypes.c_void_p),
+                ("v_pages", ctypes.c_void_p), ("block_table", ctypes.c_void_p), ("bt_stride", ctypes.c_int),
+                ("seq_of_token", ctypes.c_void_p), ("positions", ctypes.c_void_p), ("n_tokens", ctypes.c_int),
+                ("n_heads", ctypes.c_int), ("n_kv", ctypes.c_int), ("d", ctypes.c_int), ("e", ctypes.c_int),
+                ("hd_c", ctypes.c_int), ("page_size", ctypes.c_int), ("scale", ctypes.c_float),
+                ("dist_bias", ctypes.c_void_p), ("n_dist", ctypes.c_int), ("talk", ctypes.c_void_p),
+                ("head_bias", ctypes.c_void_p), ("gate", ctypes.c_void_p), ("gate_stride", ctypes.c_int),
+                ("out", ctypes.c_void_p), ("out_stride", ctypes.c_int), ("partial", ctypes.c_void_p),
+                ("n_chunks", ctypes.c_int)]
+
+
+def sigmoid_attention_chunk_keys() -> int:
+    """Keys of one chunk: the sums over keys are kept per chunk and the chunks added in order."""
+    return int(_lib.load("sigmoid_attention").fg_sigmoid_attention_chunk_keys())
+
+
+def sigmoid_attention(q: torch.Tensor, head_dim: int, out: torch.Tensor, v_head_dim: int, k_pages: torch.Tensor,
+                      v_pages: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
+                      positions: torch.Tensor, n_heads: int, scale: float,
+                      dist_bias: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None,
+                      head_bias: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                      split_for: int = 0) -> torch.Tensor:
+    """Causal attention over the paged cache whose weights are sigmoids and are not normalised over the keys.
+
+    For the query at flat row ``t`` (position ``p`` of sequence ``seq_of_token[t]``) and every key ``j <= p`` of its
+    sequence: ``s_h = q_h . k_j * scale + dist_bias[min(p - j, n_dist - 1), h]``; the heads' scores are mixed,
+    ``m_h = sum_g talk[h, g] s_g``; ``w_h = sigmoid(m_h + head_bias[h])``; ``out[t, h] = (sum_j w_h(j) v_j) *
+    sigmoid(gate[t, h])``.  ``dist_bias`` fp32 ``[n_dist, H]``, ``talk`` fp32 ``[H, H]``, ``head_bias`` fp32 ``[H]`` and
+    ``gate`` fp32 ``[T, >= H]`` may each be None.  ``q [T, >= H * head_dim]`` and ``out [T, >= H * v_head_dim]`` have
+    the cache's dtype; keys and values are read from ``k_pages [n_pages, G, P, hd]`` and ``v_pages [n_pages, G, hd,
+    P]`` (their first ``head_dim`` and ``v_head_dim`` elements).  ``split_for`` > 0: the keys of every token are
+    cut over several workgroups, enough for sequences of that many keys (for few tokens with many keys); the
+    result has the same bits either way."""
+    _gpu(q, out, k_pages, v_pages, block_table, seq_of_token, positions, dist_bias, talk, head_bias, gate)
+    T, H, d, e = q.shape[0], int(n_heads), int(head_dim), int(v_head_dim)
+    _need(k_pages.dim() == 4 and k_pages.is_contiguous(), "k_pages must be contiguous [n_pages, G, P, hd]")
+    n_pages, G, P, hd = k_pages.shape
+    _need(v_pages.is_contiguous() and v_pages.shape == (n_pages, G, hd, P) and v_pages.dtype == k_pages.dtype,
+          "v_pages must be contiguous [n_pages, G, hd, P] of k_pages' dtype")
+    _need(H > 0 and H % G == 0 and 0 < d <= hd and 0 < e <= hd and hd % 8 == 0 and P % 8 == 0,
+          "heads must be a multiple of the cache's heads, head sizes at most the cache's")
+    _need(q.dtype == k_pages.dtype and out.dtype == k_pages.dtype, "q and out must have the cache's dtype")
+    _rows_of_width(q, T, H * d, "q")
+    _rows_of_width(out, T, H * e, "out")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "block_table must be int32 [B, pages]")
+    _i32(seq_of_token, "seq_of_token", T)
+    _i32(positions, "positions", T)
+    a = _SigmoidAttentionArgs()
+    if dist_bias is not None:
+        _need(dist_bias.dtype == torch.float32 and dist_bias.is_contiguous() and dist_bias.dim() == 2
+              and dist_bias.shape[1] == H and dist_bias.shape[0] >= 1, "dist_bias must be contiguous float32 [n_dist, H]")
+        a.dist_bias, a.n_dist = dist_bias.data_ptr(), dist_bias.shape[0]
+    if talk is not None:
+        _need(talk.dtype == torch.float32 and talk.is_contiguous() and talk.shape == (H, H), "talk must be contiguous float32 [H, H]")
+        a.talk = talk.data_ptr()
+    _f32_vec(head_bias, H, "head_bias")
+    if head_bias is not None:
+        a.head_bias = head_bias.data_ptr()
+    if gate is not None:
+        _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] == T
+              and gate.shape[1] >= H, "gate must be float32 [T, >= H]")
+        a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
+    a.q, a.q_stride, a.q_hs = q.data_ptr(), q.stride(0), d
+    a.k_pages, a.v_pages, a.block_table, a.bt_stride = k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.stride(0)
+    a.seq_of_token, a.positions, a.n_tokens = seq_of_token.data_ptr(), positions.data_ptr(), T
+    a.n_heads, a.n_kv, a.d, a.e, a.hd_c, a.page_size, a.scale = H, G, d, e, hd, P, float(scale)
+    a.out, a.out_stride = out.data_ptr(), out.stride(0)
+    partial = None
+    if split_for > 0:
+        n_chunks = -(-int(split_for) // sigmoid_attention_chunk_keys())
+        if n_chunks > 1:
+            partial = torch.empty((n_chunks, T, H * e), dtype=torch.float32, device=q.device)
+            a.partial, a.n_chunks = partial.data_ptr(), n_chunks
+    st = _lib.load("sigmoid_attention").fg_sigmoid_attention(ctypes.byref(a), _code(q), _stream(q))
+    _check(st, "sigmoid_attention")
     return out

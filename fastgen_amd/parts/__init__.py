@@ -19,7 +19,7 @@ from .base import (
     unregister_part,
 )
 from . import (attention, block, embedding, feed_forward, injection, latent_attention, linear_attention, moe, norm,  # noqa: F401
-               position)  # register the built-in parts
+               position, selective_scan, sigmoid_attention)  # register the built-in parts
 
 __all__ = [
     "MATRIX", "TABLE_INT", "VECTOR", "FeedForward", "Injection", "LayerStore", "Mixer", "Norm", "PagedNeed", "Part",

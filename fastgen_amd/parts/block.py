@@ -12,6 +12,12 @@ from ..kernels.ops import ScaledRows
 from .base import FeedForward, LayerStore, Mixer, Norm, register_part
 
 
+def _no_output_bias(ffn, arrangement: str) -> None:
+    """Only an arrangement that norms a feed-forward's output adds a bias of its last projection."""
+    if ffn is not None and getattr(ffn, "bias", False):
+        raise ValueError(f"a {arrangement} layer does not take a feed-forward with biases")
+
+
 class PreNormBlock:
     """``h += mixer(norm(h)); h += ffn(norm(h))`` (``fastgen/forward.py:419-499``).
 
@@ -31,6 +37,7 @@ class PreNormBlock:
 
     def __init__(self, mixer: Mixer, ffn: FeedForward, mixer_norm: Norm, ffn_norm: Norm) -> None:
         self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
+        _no_output_bias(ffn, "pre-norm")
 
     @staticmethod
     def _run(part, x, then, *args):
@@ -67,6 +74,7 @@ class ParallelBlock:
         if ffn_norm is not None:
             raise ValueError("a parallel layer has one norm: its feed-forward reads the mixer's")
         self.mixer, self.ffn, self.mixer_norm = mixer, ffn, mixer_norm
+        _no_output_bias(ffn, "parallel")
 
     def forward(self, h: torch.Tensor, pending, ctx: Any, store: LayerStore):
         x = self.mixer_norm.forward(h, pending, ctx.act_dtype)
@@ -102,6 +110,7 @@ class SandwichBlock:
             raise ValueError("a sandwich layer needs the norms post_mixer and, with a feed-forward, ffn_norm and post_ffn")
         self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
         self.post_mixer, self.post_ffn = extra["post_mixer"], extra.get("post_ffn")
+        _no_output_bias(ffn, "sandwich")
 
     @staticmethod
     def _behind(rows, norm) -> ops.PostNormed:
@@ -117,3 +126,41 @@ class SandwichBlock:
 
 
 register_part("arrangement", "sandwich", lambda spec, *parts: SandwichBlock(*parts))
+
+
+class NormBehindBlock:
+    """``h += norm1(mixer(h)); h += norm2(ffn(h))``: the sublayers read the residual stream itself (rounded to the
+    activation dtype) and only their outputs are normed.  ``mixer_norm`` and ``ffn_norm`` are the norms behind the
+    mixer and the feed-forward.  One kernel norms what the sublayer before gave, adds it to the fp32 stream and
+    stores the stream's rows for the next sublayer.  A feed-forward whose last projection has a bias
+    (``output_bias``) leaves it to that kernel, which adds it in fp32 before the norm.  A layer without a
+    feed-forward has only the first half."""
+
+    folds_norms = False
+
+    def __init__(self, mixer: Mixer, ffn: Optional[FeedForward], mixer_norm: Norm, ffn_norm: Optional[Norm]) -> None:
+        if ffn is not None and ffn_norm is None:
+            raise ValueError("a feed-forward whose output is normed needs its norm")
+        self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
+
+    @staticmethod
+    def _stream_rows(h: torch.Tensor, pending, dtype: torch.dtype) -> torch.Tensor:
+        """Add ``pending`` to the stream and return the stream's rows in ``dtype``."""
+        x = torch.empty(h.shape, dtype=dtype, device=h.device)
+        if isinstance(pending, ops.PostNormed):
+            return ops.post_add_rmsnorm(h, pending.rows, pending.weight, pending.eps, None, 0.0, x, delta_bias=pending.bias)
+        if pending is not None:
+            ops.stream_add(h, pending, None, None)
+        return ops.post_add_rmsnorm(h, None, None, 0.0, None, 0.0, x)
+
+    def forward(self, h: torch.Tensor, pending, ctx: Any, store: LayerStore):
+        x = self._stream_rows(h, pending, ctx.act_dtype)
+        mixed = ops.PostNormed(self.mixer.forward(x, ctx, store), self.mixer_norm.weight, self.mixer_norm.eps)
+        if self.ffn is None:
+            return mixed
+        x = self._stream_rows(h, mixed, ctx.act_dtype)
+        return ops.PostNormed(self.ffn.forward(x), self.ffn_norm.weight, self.ffn_norm.eps,
+                              getattr(self.ffn, "output_bias", None))
+
+
+register_part("arrangement", "norm_behind", lambda spec, *parts: NormBehindBlock(*parts))

@@ -6,6 +6,14 @@ expert is ``W_down (silu(W_gate x) * (W_up x))`` without biases, and the output
 is the weighted sum of the chosen experts' outputs, taken in fp32.  All of it
 runs on the device (``csrc/moe.hip``): which rows went where is never looked
 at on the host, so a step with this part can be recorded.
+
+Options beyond that: ``scoring`` = ``"sigmoid"`` (an expert's score is the sigmoid
+of its logit; the chosen experts' scores divided by their sum, times
+``weight_scale``, are the weights), ``correction`` (a number per expert added to
+the scores for the choice only), ``n_groups`` / ``keep_groups`` (the experts form
+equal groups of neighbours and only those of the best groups can be chosen),
+``shared_hidden_dim`` (a gated feed-forward of that width, ``shared``, runs for
+every row and is added).
 """
 
 from __future__ import annotations
@@ -15,7 +23,8 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .base import MATRIX, VECTOR, FeedForward, TensorSpec, place, register_part
+from ..config.layout import PartSpec
+from .base import MATRIX, VECTOR, FeedForward, TensorSpec, build_part, place, register_part
 
 
 class MoE(FeedForward):
@@ -31,6 +40,25 @@ class MoE(FeedForward):
         if not 1 <= self.top <= self.n_experts:
             raise ValueError(f"{self.prefix}: top={self.top} must be between 1 and n_experts={self.n_experts}")
         self.router_bias = bool(o.get("router_bias", True))
+        self.scoring = o.get("scoring", "softmax")
+        if self.scoring not in ("softmax", "sigmoid"):
+            raise ValueError(f"{self.prefix}: scoring {self.scoring!r} is not supported ('softmax', 'sigmoid')")
+        self.has_correction = bool(o.get("correction", False))
+        self.n_groups, self.keep_groups = int(o.get("n_groups", 1)), int(o.get("keep_groups", o.get("n_groups", 1)))
+        self.weight_scale = float(o.get("weight_scale", 1.0))
+        if self.scoring != "sigmoid" and (self.has_correction or self.n_groups != 1 or self.weight_scale != 1.0):
+            raise ValueError(f"{self.prefix}: correction, groups and weight_scale go with sigmoid scoring")
+        if (self.n_groups < 1 or self.n_experts % self.n_groups or not 1 <= self.keep_groups <= self.n_groups
+                or self.top > self.keep_groups * (self.n_experts // self.n_groups)):
+            raise ValueError(f"{self.prefix}: {self.n_groups} groups of which {self.keep_groups} stay do not fit"
+                             f" {self.n_experts} experts and top={self.top}")
+        self.correction: Optional[torch.Tensor] = None
+        self.shared: Optional[FeedForward] = None
+        if o.get("shared_hidden_dim"):
+            names = o.get("names", {})
+            self.shared = build_part("feed_forward", PartSpec("swiglu", self._name("shared"), dict(
+                dim=self.dim, hidden_dim=int(o["shared_hidden_dim"]), activation="silu",
+                names={k: names[k] for k in ("gate_proj.weight", "up_proj.weight", "down_proj.weight") if k in names})))
         self.router: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
         self.w_gate: Optional[torch.Tensor] = None  # [E, hidden (padded to 8), dim]
@@ -45,6 +73,10 @@ class MoE(FeedForward):
         specs = [TensorSpec(self._name("router.weight"), (self.n_experts, self.dim), MATRIX, ("normal", 0.3))]
         if self.router_bias:
             specs.append(TensorSpec(self._name("router.bias"), (self.n_experts,), VECTOR, ("normal", 0.3)))
+        if self.has_correction:
+            specs.append(TensorSpec(self._name("correction"), (self.n_experts,), VECTOR, ("normal", 0.1)))
+        if self.shared is not None:
+            specs += self.shared.tensor_specs()
         for e in range(self.n_experts):
             specs += [TensorSpec(self._expert(e, "gate_proj.weight"), (self.hidden_dim, self.dim)),
                       TensorSpec(self._expert(e, "up_proj.weight"), (self.hidden_dim, self.dim)),
@@ -56,6 +88,10 @@ class MoE(FeedForward):
         self.router = tensors[self._name("router.weight")].to(device=device, dtype=torch.float32).contiguous()
         if self.router_bias:
             self.bias = tensors[self._name("router.bias")].to(device=device, dtype=torch.float32).contiguous()
+        if self.has_correction:
+            self.correction = tensors[self._name("correction")].to(device=device, dtype=torch.float32).contiguous()
+        if self.shared is not None:
+            self.shared.load(tensors, dtype, device)
         gate = torch.stack([tensors[self._expert(e, "gate_proj.weight")] for e in range(self.n_experts)])
         up = torch.stack([tensors[self._expert(e, "up_proj.weight")] for e in range(self.n_experts)])
         down = torch.stack([tensors[self._expert(e, "down_proj.weight")] for e in range(self.n_experts)])
@@ -90,7 +126,11 @@ class MoE(FeedForward):
         """fp32 ``[1, T, dim]``: the experts' weighted sum (plus ``plus``, rows that go to the
         residual stream with it), for a norm to add."""
         tile_rows = self.tile_rows(x.shape[0])
-        choice, weight = ops.moe_route(x, self.router, self.bias, self.top)
+        if self.shared is not None:
+            both = self.shared.forward(x)
+            plus = both if plus is None else torch.cat([t if t.dim() == 3 else t.float()[None] for t in (plus, both)])
+        choice, weight = ops.moe_route(x, self.router, self.bias, self.top, self.scoring == "sigmoid", self.correction,
+                                       self.n_groups, self.keep_groups, self.weight_scale)
         sorted_, tiles = ops.moe_sort(choice, self.n_experts, tile_rows)
         act = ops.moe_gate_up(x, self.w_gate, self.w_up, sorted_, tiles, self.top, tile_rows)
         y = ops.moe_down(act, self.w_down, sorted_, tiles, tile_rows)

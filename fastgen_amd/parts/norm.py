@@ -42,7 +42,8 @@ class RMSNorm(Norm):
         n = h.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.dim), dtype=dtype, device=h.device)
         if isinstance(delta, ops.PostNormed):
-            return ops.post_add_rmsnorm(h, delta.rows, delta.weight, delta.eps, self.weight, self.eps, out, rows)
+            return ops.post_add_rmsnorm(h, delta.rows, delta.weight, delta.eps, self.weight, self.eps, out, rows,
+                                        delta_bias=delta.bias)
         return ops.add_rmsnorm(h, delta, self.weight, self.eps, out, rows)
 
 

@@ -84,6 +84,26 @@ class Rope(PositionEncoding):
         return w.index_select(0, full.to(w.device))
 
 
+def log_bucket(distance: int, n_rows: int, far: float) -> int:
+    """The row of a table of ``n_rows`` rows that holds the bias for a key ``distance >= 0`` tokens back: one row a
+    distance below ``n_rows // 2``, then steps that grow with the logarithm of the distance and reach the last
+    row at distance ``far``."""
+    half = n_rows // 2
+    if distance < half:
+        return distance
+    return min(n_rows - 1, half + int(math.floor(math.log(distance / half) / math.log(far / half) * (n_rows - half))))
+
+
+def distance_table(rows: torch.Tensor, far: float) -> torch.Tensor:
+    """A bucketed table ``[n_rows, ...]`` spread out to one row a distance, ``[ceil(far) + 1, ...]``: every distance
+    from ``far`` on falls into the last row, so a kernel reads row ``min(distance, ceil(far))``."""
+    n_rows = rows.shape[0]
+    if n_rows < 2 or not far > n_rows // 2:
+        raise ValueError(f"a table of {n_rows} rows cannot reach its last row at distance {far}")
+    idx = [log_bucket(n, n_rows, far) for n in range(int(math.ceil(far)) + 1)]
+    return rows[torch.tensor(idx, dtype=torch.long, device=rows.device)]
+
+
 class NoPosition(PositionEncoding):
     """Positions do not enter the mixer (nothing is rotated)."""
 
