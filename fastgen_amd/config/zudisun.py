@@ -44,6 +44,7 @@ class SigmoidAttentionArgs:
     bias_max: float
     bias_rows: int
     v_mix: bool
+    vmix_stored: bool = False  # the checkpoint holds ``mix.vmix`` although the layer does not mix its values
 
 
 @dataclass(frozen=True)
@@ -116,7 +117,8 @@ class ZudisunArchitecture:
                 a = SigmoidAttentionArgs(
                     _get(m, "heads", int), _get(m, "kv_heads", int), _get(m, "dim", int), _get(m, "vdim", int),
                     _get(m, "scale", float), _get(m, "q_temp.coef", float, 0.0), _get(m, "q_temp.every", int, 0),
-                    _get(m, "bias_max", float), rows, bool(m.get("v_mix", False)))
+                    _get(m, "bias_max", float), rows, bool(m.get("v_mix", False)),
+                    shape_of is not None and shape_of(f"l{i}.mix.vmix") is not None)
                 _positive(where, heads=a.heads, kv_heads=a.kv_heads, dim=a.dim, vdim=a.vdim)
                 if a.heads % a.kv_heads:
                     raise ConfigError(f"config.json: {where}: heads={a.heads} is not a multiple of kv_heads={a.kv_heads}")
@@ -201,6 +203,7 @@ class ZudisunArchitecture:
                     dim=D, n_heads=m.heads, n_kv_heads=m.kv_heads, head_dim=m.dim, v_head_dim=m.vdim, scale=m.scale,
                     eps=eps, q_temp_coef=m.q_temp_coef, q_temp_every=m.q_temp_every, bias_far=m.bias_max,
                     bias_rows=m.bias_rows, head_mix=True, head_bias=True, head_gate=True, value_mix=m.v_mix,
+                    value_mix_stored=m.vmix_stored,
                     names={"q_proj.weight": "q", "k_proj.weight": "k", "v_proj.weight": "v", "o_proj.weight": "o",
                            "gate_proj.weight": "g", "distance_bias": "rel", "value_mix": "vmix", "head_mix": "talk",
                            "head_bias": "pb"}))

@@ -125,21 +125,29 @@ def gelu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
-def post_add_rmsnorm(h: torch.Tensor, delta: torch.Tensor, post_weight: torch.Tensor, post_eps: float,
-                     weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
-                     rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-    """``h += rmsnorm(delta) * post_weight``; with ``weight``: ``out = rmsnorm(h) * weight``.  With ``rows`` only those
-    rows, into consecutive rows of ``out``, and ``h`` stays."""
-    d = sum(_added(delta))
-    d = d * torch.rsqrt((d * d).mean(-1, keepdim=True) + post_eps) * post_weight.float()
-    s = h + d
+def post_add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], post_weight: Optional[torch.Tensor],
+                     post_eps: float, weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
+                     rows: Optional[torch.Tensor] = None, delta_bias: Optional[torch.Tensor] = None
+                     ) -> Optional[torch.Tensor]:
+    """``h += rmsnorm(delta + delta_bias) * post_weight`` (nothing without ``delta``); with ``weight``: ``out =
+    rmsnorm(h) * weight``; with ``out`` alone: ``out = h``.  With ``rows`` only those rows, into consecutive rows of
+    ``out``, and ``h`` stays."""
+    s = h
+    if delta is not None:
+        d = sum(_added(delta))
+        if delta_bias is not None:
+            d = d + delta_bias.float()
+        d = d * torch.rsqrt((d * d).mean(-1, keepdim=True) + post_eps) * post_weight.float()
+        s = h + d
     if rows is None:
         h.copy_(s)
     else:
         s = s[rows.long()]
-    if weight is None:
+    if out is None:
         return out
-    out.copy_((s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * weight.float()).to(out.dtype))
+    if weight is not None:
+        s = s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * weight.float()
+    out.copy_(s.to(out.dtype))
     return out
 
 
@@ -361,12 +369,29 @@ def gemm_skinny_qkv(x, wqkv, table: Optional[torch.Tensor], slots: torch.Tensor,
 
 
 # ------------------------------------------------------------- routed experts
-def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int,
+              sigmoid_scores: bool = False, correction: Optional[torch.Tensor] = None, n_groups: int = 1,
+              keep_groups: int = 1, weight_scale: float = 1.0):
     """The ``top`` experts with the largest fp32 logits ``x router^T + bias`` (largest first; of equal
-    logits the lower expert) and the softmax over those logits alone."""
+    logits the lower expert) and the softmax over those logits alone.  With ``sigmoid_scores``: scores
+    ``sigmoid(logit)``; chosen by score plus ``correction`` inside the ``keep_groups`` groups (of ``n_groups``) whose two
+    largest choice scores sum highest; weights: the chosen scores over their sum (+ 1e-20), times ``weight_scale``."""
     z = x.float() @ router.T + (bias if bias is not None else 0.0)
-    val, idx = torch.sort(z, dim=-1, descending=True, stable=True)
-    return idx[:, :top].to(torch.int32), torch.softmax(val[:, :top], dim=-1)
+    if not sigmoid_scores:
+        val, idx = torch.sort(z, dim=-1, descending=True, stable=True)
+        return idx[:, :top].to(torch.int32), torch.softmax(val[:, :top], dim=-1)
+    score = torch.sigmoid(z)
+    choice = score + (correction if correction is not None else 0.0)
+    T, E = choice.shape
+    if n_groups > 1 and keep_groups < n_groups:
+        per = E // n_groups
+        rank = torch.sort(choice.view(T, n_groups, per), dim=-1, descending=True).values[..., : min(2, per)].sum(-1)
+        order = torch.sort(rank, dim=-1, descending=True, stable=True).indices
+        lost = torch.zeros(T, n_groups, dtype=torch.bool, device=x.device).scatter_(1, order[:, keep_groups:], True)
+        choice = choice.masked_fill(lost[:, :, None].expand(T, n_groups, per).reshape(T, E), float("-inf"))
+    idx = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+    w = score.gather(1, idx)
+    return idx.to(torch.int32), w / (w.sum(-1, keepdim=True) + 1e-20) * weight_scale
 
 
 def moe_max_tiles(n_pairs: int, n_experts: int, tile_rows: int) -> int:
@@ -463,24 +488,32 @@ def heads_prepare(src: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
                   k_norm_dims: int = 0, v_col: int = -1, v_width: int = 0,
                   table: Optional[torch.Tensor] = None, rot_start: int = 0, rotary_dim: int = 0,
                   rotate_q: bool = True, rotate_k: bool = True, slots: Optional[torch.Tensor] = None,
-                  k_pages: Optional[torch.Tensor] = None, v_pages: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-    """Bias, a norm over the first dimensions of each head, the rotation of a run of pairs; queries to ``q_out``
-    and keys and values to their pages, every head padded with zeros to its destination's width."""
+                  k_pages: Optional[torch.Tensor] = None, v_pages: Optional[torch.Tensor] = None, norm_plain: bool = False,
+                  positions: Optional[torch.Tensor] = None, q_temp_coef: float = 0.0, q_temp_every: int = 0,
+                  v_first: Optional[torch.Tensor] = None, v_blend: float = 0.0) -> Optional[torch.Tensor]:
+    """Bias, a norm over the first dimensions of each head (``norm_plain``: also without a weight), the query's
+    temperature ``1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)``, the rotation of a run of pairs; queries to
+    ``q_out`` and keys and values (blended with ``v_first``: ``(1 - v_blend) v + v_blend v_first``) to their pages,
+    every head padded with zeros to its destination's width."""
     T = src.shape[0]
     x = src.float() + (bias.float()[None, : src.shape[1]] if bias is not None else 0.0)
 
-    def heads(col, n, width, norm_w, norm_dims, turn):
+    def heads(col, n, width, norm_w, norm_dims, turn, is_q=False):
         y = x[:, col : col + n * width].reshape(T, n, width).clone()
-        if norm_w is not None:
+        if norm_w is not None or (norm_plain and norm_dims > 0):
             part = y[..., :norm_dims]
-            y[..., :norm_dims] = part * torch.rsqrt((part * part).mean(-1, keepdim=True) + eps) * norm_w.float()[:norm_dims]
+            part = part * torch.rsqrt((part * part).mean(-1, keepdim=True) + eps)
+            y[..., :norm_dims] = part * norm_w.float()[:norm_dims] if norm_w is not None else part
+        if is_q and positions is not None and q_temp_every > 0:
+            steps = torch.div(positions.long() + 1, q_temp_every, rounding_mode="floor").float()
+            y = y * (1.0 + q_temp_coef * torch.log(steps + 1.0))[:, None, None]
         if table is not None and rotary_dim and turn:
             run = y[..., rot_start : rot_start + rotary_dim]
             y[..., rot_start : rot_start + rotary_dim] = _rotate(run, table, rotary_dim)
         return y
 
     if n_q:
-        q = heads(q_col, n_q, q_width, q_norm, q_norm_dims, rotate_q)
+        q = heads(q_col, n_q, q_width, q_norm, q_norm_dims, rotate_q, True)
         wide = torch.zeros(T, n_q, q_out_width)
         wide[..., :q_width] = q.to(q_out.dtype).float().cpu()
         q_out[:, : n_q * q_out_width] = wide.reshape(T, -1).to(q_out.dtype).to(q_out.device)
@@ -488,6 +521,8 @@ def heads_prepare(src: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
         hd = k_pages.shape[3]
         k = heads(k_col, n_kv, k_width, k_norm, k_norm_dims, rotate_k)
         v = k[..., :v_width] if v_col < 0 else x[:, v_col : v_col + n_kv * v_width].reshape(T, n_kv, v_width)
+        if v_first is not None:
+            v = (1.0 - v_blend) * v + v_blend * v_first[:, : n_kv * v_width].float().reshape(T, n_kv, v_width)
         kw, vw = torch.zeros(T, n_kv, hd), torch.zeros(T, n_kv, hd)
         kw[..., :k_width], vw[..., :v_width] = k.cpu(), v.cpu()
         _write_pages(k_pages, v_pages, slots, kw, vw)
@@ -541,4 +576,100 @@ def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.T
             a = torch.exp(torch.nn.functional.logsigmoid(zt) / tau).view(H, d)
             S.copy_(a[:, :, None] * S + k[:, :, None] * v[:, None, :])
             out[t] = torch.einsum("hde,hd->he", S, q).reshape(-1)
+    return out
+
+
+# ----------------------------------------------------- gated activation, general
+def gated_mul(gate_up: torch.Tensor, bias: Optional[torch.Tensor], activation: str, out_dtype: torch.dtype,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``act(gate + b) * (up + b)`` for rows interleaved in groups of 8 (gate, up); ``silu``, ``gelu_tanh`` or ``relu``."""
+    y = gate_up.float() + (bias.float() if bias is not None else 0.0)
+    y = y.reshape(y.shape[0], -1, 2, 8)
+    g, u = y[:, :, 0].reshape(y.shape[0], -1), y[:, :, 1].reshape(y.shape[0], -1)
+    a = torch.relu(g) if activation == "relu" else _gelu_tanh(g) if activation == "gelu_tanh" else g * torch.sigmoid(g)
+    r = (a * u).to(out_dtype)
+    if out is None:
+        return r
+    out.copy_(r)
+    return out
+
+
+# ------------------------------------------------- selective state-space recurrence
+def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, tail_off: int,
+                slot_ids: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor, out: torch.Tensor,
+                activation: Optional[str] = None) -> torch.Tensor:
+    """Per sequence: the last ``K - 1`` inputs that the state holds, then this step's, convolved per channel."""
+    C, K = taps.shape
+    for b in range(q_start.numel() - 1):
+        t0, t1 = int(q_start[b]), int(q_start[b + 1])
+        if t1 <= t0:
+            continue
+        tail = state[int(slot_ids[b]), :, tail_off : tail_off + K - 1].T  # [K - 1, C], oldest first
+        seq = torch.cat([tail.float(), x[t0:t1, :C].float()])
+        y = sum(seq[j : j + t1 - t0] * taps[:, j].float() for j in range(K))
+        if bias is not None:
+            y = y + bias.float()
+        if activation == "silu":
+            y = y * torch.sigmoid(y)
+        out[t0:t1, :C] = y.to(out.dtype)
+    return out
+
+
+def selective_scan(u: torch.Tensor, dt: torch.Tensor, dt_bias: Optional[torch.Tensor], A: torch.Tensor, bc: torch.Tensor,
+                   b_col: int, c_col: int, D: Optional[torch.Tensor], z: Optional[torch.Tensor],
+                   x_raw: Optional[torch.Tensor], taps: int, state: torch.Tensor, slot_ids: torch.Tensor,
+                   q_start: torch.Tensor, n_seqs: int, out: torch.Tensor) -> torch.Tensor:
+    """``S <- exp(d A) S + d u B``, ``y = S C + D u``, ``out = y * silu(z)`` token by token, ``d = softplus(dt + dt_bias)``; the
+    state's rows hold ``S`` and behind it the convolution's last ``taps - 1`` inputs, moved on by this step."""
+    C, N = A.shape
+    for b in range(n_seqs):
+        t0, t1 = int(q_start[b]), int(q_start[b + 1])
+        row = state[int(slot_ids[b])]
+        S = row[:, :N].clone()
+        for t in range(t0, t1):
+            d = torch.nn.functional.softplus(dt[t, :C].float() + (dt_bias if dt_bias is not None else 0.0))
+            ut = u[t, :C].float()
+            S = torch.exp(d[:, None] * A) * S + (d * ut)[:, None] * bc[t, b_col : b_col + N].float()[None, :]
+            y = S @ bc[t, c_col : c_col + N].float() + (D * ut if D is not None else 0.0)
+            if z is not None:
+                zt = z[t, :C].float()
+                y = y * zt * torch.sigmoid(zt)
+            out[t, :C] = y.to(out.dtype)
+        row[:, :N] = S
+        if taps > 1 and t1 > t0:
+            seq = torch.cat([row[:, N : N + taps - 1].T, x_raw[t0:t1, :C].float()])
+            row[:, N : N + taps - 1] = seq[-(taps - 1):].T
+    return out
+
+
+# ----------------------------------------------------------- sigmoid attention
+def sigmoid_attention(q: torch.Tensor, head_dim: int, out: torch.Tensor, v_head_dim: int, k_pages: torch.Tensor,
+                      v_pages: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
+                      positions: torch.Tensor, n_heads: int, scale: float,
+                      dist_bias: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None,
+                      head_bias: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                      split_for: int = 0) -> torch.Tensor:
+    """Token ``t`` at position ``p`` of sequence ``b`` over the keys ``0..p`` of its sequence: scores ``q . k * scale``
+    plus ``dist_bias[min(p - j, n_dist - 1), h]``, mixed over the heads by ``talk``, plus ``head_bias``; weights
+    ``sigmoid(score)``, not normalised; the heads' sums of weighted values times ``sigmoid(gate)``."""
+    H, d, e = n_heads, head_dim, v_head_dim
+    n_kv = k_pages.shape[1]
+    rep = H // n_kv
+    for t in range(q.shape[0]):
+        b, p = int(seq_of_token[t]), int(positions[t])
+        k = _gather_kv(k_pages, unpack_k, block_table[b], p + 1)[:, :, :d]
+        v = _gather_kv(v_pages, unpack_v, block_table[b], p + 1)[:, :, :e]
+        qt = q[t, : H * d].float().view(H, d)
+        s = torch.einsum("hd,jhd->hj", qt, k.repeat_interleave(rep, dim=1)) * scale  # [H, p + 1]
+        if dist_bias is not None:
+            dist = (p - torch.arange(p + 1)).clamp(max=dist_bias.shape[0] - 1)
+            s = s + dist_bias.float()[dist.to(dist_bias.device)].T
+        if talk is not None:
+            s = talk.float() @ s
+        if head_bias is not None:
+            s = s + head_bias.float()[:, None]
+        o = torch.einsum("hj,jhe->he", torch.sigmoid(s), v.repeat_interleave(rep, dim=1))
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t, :H].float())[:, None]
+        out[t, : H * e] = o.reshape(-1).to(out.dtype)
     return out

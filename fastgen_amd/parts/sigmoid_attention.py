@@ -13,8 +13,8 @@ stores ``(1 - lambda) v + lambda v_first`` in its cache, ``lambda`` a learned nu
 each other through the step's context; the first one's ``lambda`` is not used.)
 
 Options: ``dim``, ``n_heads``, ``n_kv_heads``, ``head_dim``, ``v_head_dim``, ``scale``, ``eps`` (of the unit norms),
-``q_temp_coef``, ``q_temp_every`` (0: no temperature), ``bias_far`` (None: no distance bias), ``head_mix``,
-``head_bias``, ``head_gate``, ``value_mix``.
+``q_temp_coef``, ``q_temp_every`` (0: no temperature), ``bias_far`` and ``bias_rows`` (None: no distance bias),
+``head_mix``, ``head_bias``, ``head_gate``, ``value_mix``, ``value_mix_stored``.
 """
 
 from __future__ import annotations
@@ -51,6 +51,8 @@ class SigmoidAttention(Mixer):
         self.head_bias = bool(o.get("head_bias", False))
         self.head_gate = bool(o.get("head_gate", False))
         self.value_mix = bool(o.get("value_mix", False))
+        # a layer that does not mix may still carry the number in its checkpoint: it is declared and not used
+        self.value_mix_stored = self.value_mix or bool(o.get("value_mix_stored", False))
         if self.n_heads <= 0 or self.n_kv_heads <= 0 or self.n_heads % self.n_kv_heads:
             raise ValueError(f"{self.prefix}: n_heads={self.n_heads} is not a multiple of n_kv_heads={self.n_kv_heads}")
         if self.head_dim <= 0 or self.head_dim % 2 or self.v_head_dim <= 0 or self.v_head_dim % 2:
@@ -72,7 +74,7 @@ class SigmoidAttention(Mixer):
                  TensorSpec(self._name("v_proj.weight"), (G * e, self.dim))]
         if self.bias_far is not None:
             specs.append(TensorSpec(self._name("distance_bias"), (self.bias_rows, H), VECTOR, ("normal", 0.5)))
-        if self.value_mix:
+        if self.value_mix_stored:
             specs.append(TensorSpec(self._name("value_mix"), (), VECTOR, ("normal", 0.3)))
         if self.head_mix:
             specs.append(TensorSpec(self._name("head_mix"), (H, H), VECTOR, ("normal", 0.3)))

@@ -234,3 +234,137 @@ def plain_zudisun_greedy(config: Mapping, w: Mapping[str, torch.Tensor], prompt:
     for _ in range(n_new):
         seq.append(int(plain_zudisun_forward(config, w, seq, dtype)[-1].argmax()))
     return seq[len(prompt):]
+
+
+# ------------------------------------------------------------------ shapes, weights, configurations
+def plain_zudisun_shapes(config: Mapping, bias_rows: int = 32) -> Dict[str, tuple]:
+    """The tensors of a model: name -> shape.  ``bias_rows``: rows of every distance table (a mixer's own
+    ``bias_rows`` key, if it has one, goes first)."""
+    W, out = config["width"], {}
+    out["embed"] = (config["vocab"], W)
+    for i, layer in enumerate(config["layers"]):
+        p, m = f"l{i}", layer["mixer"]
+        out[f"{p}.norm1"] = (W,)
+        if layer["type"] == "attention":
+            H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            out.update({f"{p}.mix.q": (H * d, W), f"{p}.mix.k": (G * d, W), f"{p}.mix.v": (G * e, W),
+                        f"{p}.mix.rel": (m.get("bias_rows", bias_rows), H), f"{p}.mix.talk": (H, H), f"{p}.mix.pb": (H,),
+                        f"{p}.mix.g": (H, W), f"{p}.mix.o": (W, H * e)})
+            if m.get("v_mix"):
+                out[f"{p}.mix.vmix"] = ()
+        else:
+            C, N, R, K = m["inner"], m["state"], m["dt_rank"], m["conv"]
+            out.update({f"{p}.mix.in": (2 * C, W), f"{p}.mix.conv": (C, K), f"{p}.mix.conv.b": (C,),
+                        f"{p}.mix.x": (R + 2 * N, C), f"{p}.mix.dt": (C, R), f"{p}.mix.dt.b": (C,),
+                        f"{p}.mix.A_log": (C, N), f"{p}.mix.D": (C,), f"{p}.mix.o": (W, C)})
+        mlp = layer.get("mlp")
+        if mlp is None:
+            continue
+        out[f"{p}.norm2"] = (W,)
+        if mlp["kind"] == "dense":
+            F = mlp["ff"]
+            out.update({f"{p}.mlp.gate": (F, W), f"{p}.mlp.gate.b": (F,), f"{p}.mlp.up": (F, W), f"{p}.mlp.up.b": (F,),
+                        f"{p}.mlp.down": (W, F), f"{p}.mlp.down.b": (W,)})
+        else:
+            F, E = mlp["expert"]["ff"], mlp["router"]["experts"]
+            for e_ in range(E):
+                out.update({f"{p}.mlp.e{e_}.gate": (F, W), f"{p}.mlp.e{e_}.up": (F, W), f"{p}.mlp.e{e_}.down": (W, F)})
+            out.update({f"{p}.mlp.router": (E, W), f"{p}.mlp.correction": (E,)})
+            if mlp.get("shared"):
+                S = mlp["shared"]["ff"]
+                out.update({f"{p}.mlp.shared.gate": (S, W), f"{p}.mlp.shared.up": (S, W), f"{p}.mlp.shared.down": (W, S)})
+    out["final.norm"] = (W,)
+    out["head"] = (config["vocab"], W)
+    return out
+
+
+def plain_zudisun_weights(config: Mapping, seed: int) -> Dict[str, torch.Tensor]:
+    """Random weights, representable in bfloat16, large enough that every mechanism moves the logits."""
+    g = torch.Generator().manual_seed(seed)
+    out: Dict[str, torch.Tensor] = {}
+    for name, shape in plain_zudisun_shapes(config).items():
+        r = lambda std: std * torch.randn(shape, generator=g)
+        if name.endswith(("norm1", "norm2", "norm")):
+            t = 1.0 + r(0.2)
+        elif name.endswith(".vmix"):
+            t = 0.35 + r(0.1)
+        elif name.endswith(".rel"):
+            t = r(0.7)
+        elif name.endswith(".talk"):
+            t = torch.eye(shape[0]) + r(0.25)
+        elif name.endswith(".pb"):
+            t = -2.0 + r(0.7)  # sums over hundreds of keys stay moderate
+        elif name.endswith(".A_log"):
+            t = torch.log(torch.arange(1, shape[1] + 1, dtype=torch.float32))[None, :].expand(shape) + r(0.2)
+        elif name.endswith(".dt.b"):
+            t = -2.0 + r(1.0)
+        elif name.endswith(".D"):
+            t = 1.0 + r(0.3)
+        elif name.endswith(".correction"):
+            t = r(0.3)
+        elif name.endswith(".conv"):
+            t = r(0.5)
+        elif name.endswith(".b"):
+            t = r(0.3)
+        elif name.endswith(".router"):
+            t = r(4.0 / math.sqrt(shape[-1]))
+        elif name == "embed":
+            t = r(1.0)
+        else:
+            t = r(1.5 / math.sqrt(shape[-1]))
+        out[name] = t.to(torch.bfloat16).float()
+    return out
+
+
+def _sig(H, G, d, e, every=16, coef=0.5, far=40, v_mix=False, rows=None):
+    m = {"heads": H, "kv_heads": G, "dim": d, "vdim": e, "scale": d ** -0.5, "q_temp": {"coef": coef, "every": every},
+         "bias_max": far, "v_mix": v_mix}
+    if rows is not None:
+        m["bias_rows"] = rows
+    return m
+
+
+def _scan(C, N, R, K):
+    return {"inner": C, "state": N, "dt_rank": R, "conv": K}
+
+
+def _moe(E, top, F, groups=1, keep=1, scale=1.0, shared=None):
+    return {"kind": "moe", "expert": {"ff": F}, "router": {"experts": E, "top": top, "scale": scale,
+                                                             "groups": {"count": groups, "keep": keep}},
+            "shared": None if shared is None else {"ff": shared}}
+
+
+def _zconfig(width, vocab, layers, eps=1e-5):
+    return {"architecture": "Zudisun", "width": width, "vocab": vocab, "norm": {"eps": eps}, "layers": layers}
+
+
+# both mixers, both feed-forwards, a layer without one; values mixed over three layers; tables of 12 rows
+PAIR = _zconfig(64, 97, [
+    {"type": "mamba1", "mixer": _scan(96, 8, 6, 4), "mlp": _moe(6, 2, 40, groups=3, keep=2, scale=2.0, shared=48)},
+    {"type": "attention", "mixer": _sig(4, 2, 32, 16, far=30, v_mix=True, rows=12), "mlp": {"kind": "dense", "ff": 96}},
+    {"type": "attention", "mixer": _sig(2, 2, 16, 16, every=5, coef=1.5, far=100, v_mix=True, rows=12), "mlp": None},
+    {"type": "mamba1", "mixer": _scan(80, 16, 4, 2), "mlp": {"kind": "dense", "ff": 72}},
+    {"type": "attention", "mixer": _sig(6, 2, 16, 16, every=64, far=13, v_mix=True, rows=12), "mlp": _moe(4, 1, 56)},
+])
+# one layer of a kind each, for tests of a mechanism inside the engine
+ONLY_SIGMOID = _zconfig(48, 61, [{"type": "attention", "mixer": _sig(2, 1, 16, 24, every=7, far=50, rows=16),
+                                  "mlp": {"kind": "dense", "ff": 56}}])
+ONLY_SCAN = _zconfig(48, 61, [{"type": "mamba1", "mixer": _scan(64, 12, 5, 3), "mlp": None}])
+# sizes that are no multiples of 8 or 16, head counts that are no powers of two, one kv head for all and one a
+# head, values wider than keys, one tap and many taps, a state of one and of many values, a step rank of one,
+# tables with an odd number of rows, a far distance beyond every prompt and one just past half of the table,
+# a temperature that changes at every position and one that never does, every expert chosen, a group an
+# expert, no shared expert, groups of which all stay, a mixing layer between layers that do not mix
+ODD = _zconfig(100, 101, [
+    {"type": "attention", "mixer": _sig(5, 5, 20, 12, every=1, coef=0.25, far=1000.0, rows=9), "mlp": _moe(3, 3, 36, scale=0.5)},
+    {"type": "mamba1", "mixer": _scan(70, 1, 1, 1), "mlp": None},
+    {"type": "attention", "mixer": _sig(7, 1, 10, 26, every=100000, far=5, v_mix=True, rows=7), "mlp": {"kind": "dense", "ff": 36}},
+    {"type": "mamba1", "mixer": _scan(36, 37, 9, 9), "mlp": _moe(8, 2, 20, groups=8, keep=3, shared=28)},
+    {"type": "attention", "mixer": _sig(3, 1, 10, 26, every=3, coef=2.0, far=64.5, v_mix=True, rows=7), "mlp": _moe(6, 4, 24, groups=2, keep=2)},
+    {"type": "attention", "mixer": _sig(34, 2, 8, 8, far=33, rows=64), "mlp": None},
+], eps=1e-4)
+# recurrent layers alone: a model without a cache of keys
+NO_CACHE = _zconfig(56, 83, [
+    {"type": "mamba1", "mixer": _scan(48, 4, 3, 5), "mlp": {"kind": "dense", "ff": 64}},
+    {"type": "mamba1", "mixer": _scan(112, 20, 8, 2), "mlp": _moe(5, 2, 32, shared=16)},
+])
