@@ -7,6 +7,7 @@
     python bench.py --workload readme --shape 70b   # the same load at the 70B sizes, cache = the memory left
     python bench.py --workload buderax      # the Buderax design beside the dense Llama at equal sizes
     python bench.py --workload gisodra      # the Gisodra design beside the dense Llama at equal sizes
+    python bench.py --workload zudisun      # the Zudisun design beside Gisodra and the dense Llama at equal sizes
 
 The model has the layer sizes of Llama 3.1 8B (32 layers, hidden 4096, 32
 heads, 8 kv heads, head size 128, feed-forward 14336, vocabulary 128256,
@@ -473,6 +474,196 @@ def gisodra_workload(prefill_tokens: int = 2048, batch: int = 8, context: int = 
     return 0
 
 
+# Zudisun at sizes that resemble a real model's layers: eight layers in the order sigmoid attention with a dense
+# feed-forward, selective scan with a routed one, selective scan with a dense one, sigmoid attention with a routed
+# one, twice.  Beside it: Gisodra (the framework's other design with attention and recurrent layers side by side)
+# and the dense Llama, both of the same width, heads, head size, dense feed-forward width and number of layers.
+ZUDISUN_SIZES = {
+    "w1024": dict(width=1024, heads=16, kv_heads=4, dim=64, ff=2816, inner=2048, state=16, dt_rank=64, conv=4,
+                  experts=16, top=2, expert_ff=704, groups=4, keep=2, shared_ff=704, far=2048.0, rows=32, vocab=32000),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=5632, inner=4096, state=16, dt_rank=128, conv=4,
+                  experts=32, top=4, expert_ff=768, groups=8, keep=4, shared_ff=1536, far=2048.0, rows=32, vocab=32000),
+}
+
+
+def _zudisun_configs(z: dict):
+    attn = lambda mlp: dict(type="attention", mlp=mlp, mixer=dict(
+        heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5,
+        q_temp=dict(coef=0.5, every=512), bias_max=z["far"], bias_rows=z["rows"], v_mix=True))
+    scan = lambda mlp: dict(type="mamba1", mlp=mlp, mixer=dict(inner=z["inner"], state=z["state"], dt_rank=z["dt_rank"], conv=z["conv"]))
+    dense_ff = dict(kind="dense", ff=z["ff"])
+    routed = dict(kind="moe", expert=dict(ff=z["expert_ff"]), shared=dict(ff=z["shared_ff"]),
+                  router=dict(experts=z["experts"], top=z["top"], scale=1.5, groups=dict(count=z["groups"], keep=z["keep"])))
+    layers = [attn(dense_ff), scan(routed), scan(dense_ff), attn(routed)] * 2
+    new = dict(architecture="Zudisun", width=z["width"], vocab=z["vocab"], norm=dict(eps=1e-6), layers=layers)
+    dense = dict(architectures=["LlamaForCausalLM"], hidden_size=z["width"], intermediate_size=z["ff"],
+                 num_hidden_layers=len(layers), num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"],
+                 rms_norm_eps=1e-6, vocab_size=z["vocab"], rope_theta=500000.0, rope_scaling=None,
+                 tie_word_embeddings=False, max_position_embeddings=131072)
+    return new, dense
+
+
+def _zudisun_kernels(z: dict, rows: int, context: int) -> dict:
+    """The design's own kernels at ``rows`` tokens (one prompt of ``rows`` tokens, or ``rows`` sequences of one token
+    at ``context`` cached ones), each beside the like kernel of the framework's other models on operands of the
+    same size: microseconds, and the shares of the memory roofline (the bytes the kernel has to move), of the
+    matrix cores' (its products' flops) and of the fp32 vector units' (the flops that are fp32 by design)."""
+    import torch
+
+    from fastgen_amd.kernels import ops
+    from fastgen_amd.parts.position import distance_table
+
+    D, H, G, d, P = z["width"], z["heads"], z["kv_heads"], z["dim"], PAGE
+    C, N, R, K = z["inner"], z["state"], z["dt_rank"], z["conv"]
+    g = torch.Generator(device="cuda").manual_seed(rows)
+    rnd = lambda *shape: (torch.randn(*shape, generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+    f32 = lambda *shape: torch.randn(*shape, generator=g, device="cuda")
+    i32 = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
+    decode = rows <= 64
+    n_seqs = rows if decode else 1
+    out = {}
+
+    def put(name, fn, nbytes, flops=0, vector_flops=0):
+        t = _time(fn)
+        out[name] = {"us": round(t * 1e6, 1), "hbm_frac": round(nbytes / t / PEAK_HBM, 4),
+                     "mfma_frac": round(flops / t / PEAK_FLOPS["bf16"], 4),
+                     "fp32_vector_frac": round(vector_flops / t / PEAK_FLOPS["fp32"], 4)}
+
+    # ---- attention over the pages: a prompt of `rows` tokens, or `rows` sequences of `context` keys each
+    per_seq = rows if not decode else context
+    pages_per_seq = -(-per_seq // P)
+    n_pages = n_seqs * pages_per_seq + 1
+    kp, vp = rnd(n_pages, G, P, d), rnd(n_pages, G, d, P)
+    table = torch.arange(n_seqs * pages_per_seq, dtype=torch.int32, device="cuda").view(n_seqs, pages_per_seq).contiguous()
+    if decode:
+        seq_of_token, positions = i32(list(range(rows))), i32([context - 1] * rows)
+        pairs = rows * context
+    else:
+        seq_of_token, positions = i32([0] * rows), i32(list(range(rows)))
+        pairs = rows * (rows + 1) // 2
+    q, o = rnd(rows, H * d), torch.empty(rows, H * d, dtype=torch.bfloat16, device="cuda")
+    rel = distance_table(f32(z["rows"], H), z["far"]).contiguous()
+    talk, pb, gate = f32(H, H) / H, f32(H) - 3.0, f32(rows, H)
+    split = per_seq if decode else 0
+    kv_bytes = (n_seqs * per_seq * 2 * G * d + 2 * rows * H * d) * 2
+    # per (query, key) pair: the two products (matrix cores), and in fp32 by design: the heads' mixing (2 H^2), the
+    # bias, scale and sigmoid (about 8 a head)
+    put("sigmoid_attention", lambda: ops.sigmoid_attention(q, d, o, d, kp, vp, table, seq_of_token, positions, H, d ** -0.5, rel,
+                                                           talk, pb, gate, split_for=split),
+        kv_bytes, 4 * pairs * H * d, pairs * (2 * H * H + 8 * H))
+    put("sigmoid_attention, heads not mixed", lambda: ops.sigmoid_attention(q, d, o, d, kp, vp, table, seq_of_token, positions, H,
+                                                                            d ** -0.5, rel, None, pb, gate, split_for=split),
+        kv_bytes, 4 * pairs * H * d, pairs * 8 * H)
+    q_start = i32(list(range(0, rows + 1, rows // n_seqs)))
+    put("paged_attention_general (the softmax attention's general kernel)",
+        lambda: ops.paged_attention_general(q, o, kp, vp, table, seq_of_token, positions, H, d ** -0.5), kv_bytes, 4 * pairs * H * d)
+    # ---- between the q/k/v product and the attention: unit norms, temperature, blended values, cache write
+    width = (H + 2 * G) * d + H
+    rows32, v_first = f32(rows, width), f32(rows, G * d)
+    slots = torch.arange(rows, dtype=torch.int32, device="cuda") if not decode else i32([b * pages_per_seq * P + context - 1 for b in range(rows)])
+    put("heads_prepare (unit norms, temperature, blend)", lambda: ops.heads_prepare(
+        rows32, None, 1e-6, n_q=H, q_col=0, q_width=d, q_norm_dims=d, q_out=q, q_out_width=d, n_kv=G, k_col=H * d, k_width=d,
+        k_norm_dims=d, v_col=(H + G) * d, v_width=d, slots=slots, k_pages=kp, v_pages=vp, norm_plain=True, positions=positions,
+        q_temp_coef=0.5, q_temp_every=512, v_first=v_first, v_blend=0.3), rows * (width * 4 + G * d * 4 + (H + 2 * G) * d * 2))
+    nw = f32(d)
+    put("heads_prepare (gisodra: norms with weights)", lambda: ops.heads_prepare(
+        rows32, None, 1e-6, n_q=H, q_col=0, q_width=d, q_norm=nw, q_norm_dims=d, q_out=q, q_out_width=d, n_kv=G, k_col=H * d,
+        k_width=d, k_norm=nw, k_norm_dims=d, v_col=(H + G) * d, v_width=d, slots=slots, k_pages=kp, v_pages=vp),
+        rows * (width * 4 + (H + 2 * G) * d * 2))
+    # ---- the selective scan and its convolution; beside Gisodra's recurrence with a state of the same size
+    xz, dt = rnd(rows, 2 * C), f32(rows, C)
+    narrow = rnd(rows, -(-(R + 2 * N) // 8) * 8)
+    taps, cb, db, A, Dk = f32(C, K), f32(C), f32(C) - 2.0, -f32(C, N).abs() - 0.1, f32(C)
+    state = torch.zeros(n_seqs + 1, C, N + K - 1, device="cuda")
+    slot_ids = torch.arange(n_seqs, dtype=torch.int32, device="cuda")
+    seq_rows = i32([t // (rows // n_seqs) for t in range(rows)])
+    u, y = torch.empty(rows, C, dtype=torch.bfloat16, device="cuda"), torch.empty(rows, C, dtype=torch.bfloat16, device="cuda")
+    put("causal_conv", lambda: ops.causal_conv(xz, taps, cb, state, N, slot_ids, seq_rows, q_start, u, activation="silu"),
+        rows * C * 4 + n_seqs * C * (K - 1) * 4, 0, 2 * rows * C * K)
+    # per state element and token: a product and an exponential for the decay, two multiply-adds; all fp32 by design
+    put("selective_scan", lambda: ops.selective_scan(u, dt, db, A, narrow, R, R + N, Dk, xz[:, C:], xz, K, state, slot_ids, q_start,
+                                                     n_seqs, y),
+        2 * n_seqs * C * (N + K - 1) * 4 + rows * (C * (2 + 4 + 2 + 2 + 2) + 2 * N * 2), 0, 6 * rows * C * N)
+    gh, gd = z["heads"], 64
+    ge = C * N // (gh * gd)  # as many state elements as the scan has
+    gw = 2 * gh * gd + 2 * gh * ge
+    rows16, zz, zb = rnd(rows, gw), f32(rows, gh * gd), f32(gh * gd)
+    gstate = torch.zeros(n_seqs + 1, gh, gd, ge, device="cuda")
+    o32 = torch.empty(rows, gh * ge, device="cuda")
+    q_start_host = q_start.cpu().numpy()
+    t = _time(lambda: ops.decay_scan(rows16, 0, gh * gd, 2 * gh * gd, zz, zb, 16.0, gd ** -0.5, gstate, slot_ids, q_start, n_seqs, o32,
+                                     q_start_host=q_start_host))
+    out["decay_scan (gisodra, a state of equal size)"] = {
+        "us": round(t * 1e6, 1),
+        "hbm_frac": round((2 * n_seqs * gh * gd * ge * 4 + rows * (gw * 2 + gh * gd * 4 + gh * ge * 4)) / t / PEAK_HBM, 4),
+        "fp32_vector_frac": round(4 * rows * gh * gd * ge / t / PEAK_FLOPS["fp32"], 4)}
+    if not decode:
+        t = _time(lambda: ops.decay_scan(rows16, 0, gh * gd, 2 * gh * gd, zz, zb, 16.0, gd ** -0.5, gstate, slot_ids, q_start, n_seqs, o32))
+        out["decay_scan (gisodra), token by token"] = {"us": round(t * 1e6, 1),
+                                                        "fp32_vector_frac": round(4 * rows * gh * gd * ge / t / PEAK_FLOPS["fp32"], 4)}
+    # ---- the dense feed-forward's activation with biases; beside the activation alone
+    F = z["ff"]
+    gu, b = f32(rows, 2 * F), f32(2 * F)
+    put("gated_mul (relu, biases, fp32 rows)", lambda: ops.gated_mul(gu, b, "relu", torch.bfloat16), rows * F * (8 + 2))
+    gu16 = rnd(rows, 2 * F)
+    put("silu_mul (llama, bf16 rows)", lambda: ops.silu_mul(gu16), rows * F * (4 + 2))
+    # ---- the stream's rows with a sublayer's normed output added; beside the dense decoder's norm
+    h, delta, w1, w2, ob = f32(rows, D), rnd(rows, D), rnd(D), rnd(D), f32(D)
+    normed = torch.empty(rows, D, dtype=torch.bfloat16, device="cuda")
+    put("post_add_rmsnorm (rows of the stream, output bias)",
+        lambda: ops.post_add_rmsnorm(h, delta, w1, 1e-6, None, 0.0, normed, delta_bias=ob), rows * D * (4 + 4 + 2 + 2))
+    put("add_rmsnorm (llama)", lambda: ops.add_rmsnorm(h, delta, w2, 1e-6, normed), rows * D * (4 + 4 + 2 + 2))
+    # ---- the router: sigmoid scores, groups, correction; beside the softmax router
+    x, wr, corr = rnd(rows, D), f32(z["experts"], D) / 30, f32(z["experts"])
+    route_bytes = rows * D * 2 + z["experts"] * D * 4
+    put("moe_route (sigmoid, groups)", lambda: ops.moe_route(x, wr, None, z["top"], True, corr, z["groups"], z["keep"], 1.5),
+        route_bytes, 0, 2 * rows * D * z["experts"])
+    put("moe_route (buderax, softmax)", lambda: ops.moe_route(x, wr, None, z["top"]), route_bytes, 0, 2 * rows * D * z["experts"])
+    return out
+
+
+def zudisun_workload(prefill_tokens: int = 2048, batch: int = 8, context: int = 1024, steps: int = 32, warmup: int = 8) -> int:
+    """Prefill and decode throughput of Zudisun models with random bfloat16 weights beside Gisodra and dense Llama
+    models of equal sizes, and the design's own kernels beside the other models' like ones.  One JSON line."""
+    import torch
+
+    from fastgen_amd.engine import Engine
+
+    results = {}
+    for name, z in ZUDISUN_SIZES.items():
+        new, dense = _zudisun_configs(z)
+        hybrid, _ = _gisodra_configs(GISODRA_SIZES[name])
+        row = {"layers": len(new["layers"])}
+        for label, cfg in (("zudisun", new), ("gisodra", hybrid), ("llama", dense)):
+            engine = Engine.from_config(cfg, seed=5, dtype=torch.bfloat16, page_size=PAGE,
+                                        max_tokens=max(batch * (context + 256), prefill_tokens + PAGE), max_batch=batch,
+                                        max_step_tokens=prefill_tokens)
+            g = torch.Generator().manual_seed(0)
+            prompt = lambda n: torch.randint(0, z["vocab"], (n,), generator=g).tolist()
+            pre = min(engine.time_prefill(prompt(prefill_tokens), repeats=5))
+            dt = engine.time_decode([prompt(context) for _ in range(batch)], steps=steps, warmup=warmup)
+            row[label] = {"prefill_tok_s": round(prefill_tokens / pre, 1), "prefill_ms": round(pre * 1e3, 3),
+                          "decode_tok_s": round(batch * steps / dt, 1), "decode_ms_per_step": round(dt / steps * 1e3, 4),
+                          "weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
+            print(f"[bench] {name} {label}: {row[label]}", file=sys.stderr, flush=True)
+            del engine
+            torch.cuda.empty_cache()
+        row["kernels_prefill"] = _zudisun_kernels(z, prefill_tokens, context)
+        row["kernels_decode"] = _zudisun_kernels(z, batch, context)
+        print(f"[bench] {name} kernels: {row['kernels_prefill']} {row['kernels_decode']}", file=sys.stderr, flush=True)
+        results[name] = row
+    first = results[next(iter(results))]
+    print(json.dumps({
+        "metric": "Zudisun beside Gisodra and the dense Llama at equal sizes: prefill and decode tok/s", "unit": "tokens/s",
+        "value": first["zudisun"]["decode_tok_s"], "n_gpus": 1, "steps": steps, "warmup": warmup, "higher_is_better": True,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"prefill_tokens": prefill_tokens, "decode_batch": batch, "decode_context": context, "page_size": PAGE,
+                   "sizes": ZUDISUN_SIZES},
+        "results": results,
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -490,10 +681,10 @@ def main() -> int:
                          " 2,048); more are fed untimed, in portions")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
-    ap.add_argument("--workload", choices=["decode", "serve", "readme", "buderax", "gisodra"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "serve", "readme", "buderax", "gisodra", "zudisun"], default="decode",
                     help="decode (default): the step benchmark; serve: continuous batching of 256 requests; "
-                         "readme: the load of the reference's README; buderax, gisodra: that design beside the dense "
-                         "Llama at equal sizes")
+                         "readme: the load of the reference's README; buderax, gisodra, zudisun: that design beside the "
+                         "dense Llama at equal sizes")
     ap.add_argument("--step-budget", type=int, default=2048, help="tokens a step of the serve workload")
     ap.add_argument("--show-choices", action="store_true",
                     help="print (stderr) which kernel the run's measurements chose for each matrix product")
@@ -507,6 +698,8 @@ def main() -> int:
         return readme_workload(a.shape or "8b")
     if a.workload == "gisodra":
         return gisodra_workload(prefill_tokens=a.prefill_tokens, batch=a.batch, steps=min(a.steps, 32), warmup=a.warmup)
+    if a.workload == "zudisun":
+        return zudisun_workload(prefill_tokens=a.prefill_tokens, batch=a.batch, steps=min(a.steps, 32), warmup=a.warmup)
     if a.workload == "buderax":
         return buderax_workload(prefill_tokens=a.prefill_tokens, batch=a.batch, steps=min(a.steps, 32), warmup=a.warmup)
     a.shape = a.shape or "8b"

@@ -99,7 +99,7 @@ def plain_sigmoid_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, s
     rows = rel.shape[0]
     idx = torch.tensor([[plain_bucket(i - j, rows, far) if j <= i else 0 for j in range(T)] for i in range(T)])
     s = s + _hi(rel)[idx].permute(2, 0, 1)
-    s = torch.einsum("hg,gij->hij", _hi(talk), s) + _hi(head_bias)[:, None, None]
+    s = torch.einsum("hg,gij->hij", talk.to(s.dtype), s) + _hi(head_bias)[:, None, None]
     wgt = torch.sigmoid(s) * torch.tril(torch.ones(T, T, dtype=s.dtype))
     return torch.einsum("hij,jhe->ihe", wgt, v.repeat_interleave(rep, dim=1))
 
@@ -169,7 +169,7 @@ def plain_mamba_mixer(x: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, m:
 def plain_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int,
                 scale: float):
     """Per row of ``x [T, width]``: the chosen experts ``[T, top]`` and their weights."""
-    s = torch.sigmoid(_hi(x) @ _hi(router).T)
+    s = torch.sigmoid(_hi(x) @ router.to(_hi(x).dtype).T)
     choice = s + _hi(correction)
     T, E = s.shape
     per = E // groups
