@@ -581,8 +581,9 @@ def _zudisun_kernels(z: dict, rows: int, context: int) -> dict:
     put("causal_conv", lambda: ops.causal_conv(xz, taps, cb, state, N, slot_ids, seq_rows, q_start, u, activation="silu"),
         rows * C * 4 + n_seqs * C * (K - 1) * 4, 0, 2 * rows * C * K)
     # per state element and token: a product and an exponential for the decay, two multiply-adds; all fp32 by design
+    q_start_host = q_start.cpu().numpy()  # (with it, long runs of tokens are scanned in chunks side by side)
     put("selective_scan", lambda: ops.selective_scan(u, dt, db, A, narrow, R, R + N, Dk, xz[:, C:], xz, K, state, slot_ids, q_start,
-                                                     n_seqs, y),
+                                                     n_seqs, y, q_start_host=q_start_host),
         2 * n_seqs * C * (N + K - 1) * 4 + rows * (C * (2 + 4 + 2 + 2 + 2) + 2 * N * 2), 0, 6 * rows * C * N)
     gh, gd = z["heads"], 64
     ge = C * N // (gh * gd)  # as many state elements as the scan has
@@ -590,7 +591,6 @@ def _zudisun_kernels(z: dict, rows: int, context: int) -> dict:
     rows16, zz, zb = rnd(rows, gw), f32(rows, gh * gd), f32(gh * gd)
     gstate = torch.zeros(n_seqs + 1, gh, gd, ge, device="cuda")
     o32 = torch.empty(rows, gh * ge, device="cuda")
-    q_start_host = q_start.cpu().numpy()
     t = _time(lambda: ops.decay_scan(rows16, 0, gh * gd, 2 * gh * gd, zz, zb, 16.0, gd ** -0.5, gstate, slot_ids, q_start, n_seqs, o32,
                                      q_start_host=q_start_host))
     out["decay_scan (gisodra, a state of equal size)"] = {
@@ -598,6 +598,8 @@ def _zudisun_kernels(z: dict, rows: int, context: int) -> dict:
         "hbm_frac": round((2 * n_seqs * gh * gd * ge * 4 + rows * (gw * 2 + gh * gd * 4 + gh * ge * 4)) / t / PEAK_HBM, 4),
         "fp32_vector_frac": round(4 * rows * gh * gd * ge / t / PEAK_FLOPS["fp32"], 4)}
     if not decode:
+        put("selective_scan, token by token", lambda: ops.selective_scan(u, dt, db, A, narrow, R, R + N, Dk, xz[:, C:], xz, K, state,
+                                                                         slot_ids, q_start, n_seqs, y), 0, 0, 6 * rows * C * N)
         t = _time(lambda: ops.decay_scan(rows16, 0, gh * gd, 2 * gh * gd, zz, zb, 16.0, gd ** -0.5, gstate, slot_ids, q_start, n_seqs, o32))
         out["decay_scan (gisodra), token by token"] = {"us": round(t * 1e6, 1),
                                                         "fp32_vector_frac": round(4 * rows * gh * gd * ge / t / PEAK_FLOPS["fp32"], 4)}

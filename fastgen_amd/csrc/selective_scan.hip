@@ -14,6 +14,9 @@
 //                  (grid.y: the sequence), with the next token's operands in flight while one is computed.
 //                  When it is done it stores the state and moves the convolution's tail on by this step's
 //                  tokens (`x_raw`: the convolution's input rows), so the next step finds both.
+//  Long prompts are scanned in chunks of tokens side by side, in three passes: every chunk from a zero state
+//  (no outputs; what it adds to the state and the sum of its step sizes are kept), then the state that every
+//  chunk starts from (scan_chunk_states), then every chunk from that state with its outputs.
 //
 // All arithmetic is fp32; the state never leaves fp32.  What a token gets depends on its sequence's earlier
 // tokens alone, in their order: not on the batch and not on how the tokens were cut into steps.
@@ -63,6 +66,7 @@ extern "C" int fg_causal_conv(const void* x, int ldx, const float* taps, const f
   else if (src_dtype == FG_F32 && act_dtype == FG_BF16) GO(float, bf16_t);
   else return FG_ERR_ARG;
 #undef GO
+#undef GO_OUT
   return fg_launch_status();
 }
 
@@ -79,6 +83,8 @@ struct ScanArgs {
   const int* slot_ids; const int* q_start;
   void* out; int ldo;              // [T, >= C] activation dtype
   int C, N, K, LP;
+  int write_out, write_state, write_tail;  // what a pass leaves behind (all three: the whole step in one pass)
+  float* dsum;                     // [n_seqs, C] or null: the sum of a sequence's step sizes, per channel
 };
 
 template <class TA> __device__ __forceinline__ float fast_exp(float x);
@@ -86,7 +92,7 @@ template <> __device__ __forceinline__ float fast_exp<float>(float x) { return e
 // bfloat16 operands: the hardware's exponential (a few ulp of 32-bit)
 template <> __device__ __forceinline__ float fast_exp<bf16_t>(float x) { return __expf(x); }
 
-template <class TA, class TD, int SPL>
+template <class TA, class TD, int SPL, bool OUT>
 __global__ __launch_bounds__(SS_THREADS) void selective_scan_kernel(const ScanArgs a) {
   const int tid = blockIdx.x * SS_THREADS + threadIdx.x;
   const int c = tid / a.LP, g = tid % a.LP;
@@ -125,7 +131,8 @@ __global__ __launch_bounds__(SS_THREADS) void selective_scan_kernel(const ScanAr
       n_C[i] = in ? to_f<TA>(Cp[(size_t)t * a.ldbc + i]) : 0.f;
     }
   };
-  fetch(t0);
+  float d_total = 0.f;
+  if (t0 < t1) fetch(t0);
   for (int t = t0; t < t1; ++t) {
     const float uv = n_u, zv = n_z;
     float d = n_dt + bias;
@@ -134,25 +141,31 @@ __global__ __launch_bounds__(SS_THREADS) void selective_scan_kernel(const ScanAr
     for (int i = 0; i < SPL; ++i) { Bv[i] = n_B[i]; Cv[i] = n_C[i]; }
     if (t + 1 < t1) fetch(t + 1);
     d = d > 20.f ? d : log1pf(expf(d));  // softplus
+    d_total += d;
     const float du = d * uv;
     float y = 0.f;
 #pragma unroll
     for (int i = 0; i < SPL; ++i) {
       S[i] = fast_exp<TA>(d * An[i]) * S[i] + du * Bv[i];
-      y = fmaf(S[i], Cv[i], y);
+      if (OUT) y = fmaf(S[i], Cv[i], y);
     }
-    for (int m = 1; m < a.LP; m <<= 1) y += __shfl_xor(y, m, FG_WAVE);
-    if (g == 0 && live) {
-      y = fmaf(skip, uv, y);
-      if (z) y *= zv / (1.f + fast_exp<TA>(-zv));
-      out[(size_t)t * a.ldo] = from_f<TA>(y);
+    if (OUT) {
+      for (int m = 1; m < a.LP; m <<= 1) y += __shfl_xor(y, m, FG_WAVE);
+      if (g == 0 && live) {
+        y = fmaf(skip, uv, y);
+        if (z) y *= zv / (1.f + fast_exp<TA>(-zv));
+        out[(size_t)t * a.ldo] = from_f<TA>(y);
+      }
     }
   }
   if (!live) return;
+  if (a.write_state) {
 #pragma unroll
-  for (int i = 0; i < SPL; ++i)
-    if (n0 + i < a.N) row[n0 + i] = S[i];
-  if (g == 0 && a.K > 1) {
+    for (int i = 0; i < SPL; ++i)
+      if (n0 + i < a.N) row[n0 + i] = S[i];
+  }
+  if (a.dsum && g == 0) a.dsum[(size_t)b * a.C + cc] = d_total;
+  if (g == 0 && a.K > 1 && a.write_tail) {
     // the convolution's tail: the last K - 1 inputs of the sequence, old ones where this step brought fewer
     float* tail = row + a.N;
     const int L = t1 - t0, keep = a.K - 1;
@@ -181,16 +194,83 @@ extern "C" int fg_selective_scan(const ScanArgs* args, int n_seqs, int dt_dtype,
   if (a.LP < 1 || a.LP > 64 || (a.LP & (a.LP - 1)) || a.LP * spl < a.N) return FG_ERR_ARG;
   const long long threads = (long long)a.C * a.LP;
   dim3 grid((unsigned)((threads + SS_THREADS - 1) / SS_THREADS), n_seqs);
-#define GO(TA, TD)                                                                      \
-  do {                                                                                  \
-    if (spl == 4) selective_scan_kernel<TA, TD, 4><<<grid, SS_THREADS, 0, stream>>>(a); \
-    else if (spl == 8) selective_scan_kernel<TA, TD, 8><<<grid, SS_THREADS, 0, stream>>>(a); \
-    else selective_scan_kernel<TA, TD, 16><<<grid, SS_THREADS, 0, stream>>>(a);         \
+#define GO_OUT(TA, TD, OUT)                                                                          \
+  do {                                                                                               \
+    if (spl == 4) selective_scan_kernel<TA, TD, 4, OUT><<<grid, SS_THREADS, 0, stream>>>(a);        \
+    else if (spl == 8) selective_scan_kernel<TA, TD, 8, OUT><<<grid, SS_THREADS, 0, stream>>>(a);   \
+    else selective_scan_kernel<TA, TD, 16, OUT><<<grid, SS_THREADS, 0, stream>>>(a);                \
+  } while (0)
+#define GO(TA, TD)                                      \
+  do {                                                  \
+    if (a.write_out) GO_OUT(TA, TD, true);              \
+    else GO_OUT(TA, TD, false);                         \
   } while (0)
   if (act_dtype == FG_F32 && dt_dtype == FG_F32) GO(float, float);
   else if (act_dtype == FG_BF16 && dt_dtype == FG_F32) GO(bf16_t, float);
   else if (act_dtype == FG_BF16 && dt_dtype == FG_BF16) GO(bf16_t, bf16_t);
   else return FG_ERR_ARG;
 #undef GO
+#undef GO_OUT
+  return fg_launch_status();
+}
+
+// Long runs of tokens, scanned chunk by chunk: after every chunk was scanned from a zero state (its rows of
+// `chunks` hold what it adds, `dsum` the sums of its step sizes), the state that each chunk starts from.  Over
+// a chunk the decay of S[c, n] is exp(A[c, n] * dsum[c]).  Per sequence b with the chunks seq_chunk[b] ..
+// seq_chunk[b+1]-1, in their order:  start_0 = state[slot];  start_{k+1} = exp(A dsum_k) start_k + chunks_k.
+// chunks_k becomes start_k, and the state's row what the last chunk leaves.  A thread a (channel, state value).
+// The convolution's tail moves on by the sequence's tokens (as the scan does it in one pass).
+template <class TA>
+__global__ __launch_bounds__(SS_THREADS) void scan_chunk_states_kernel(
+    float* __restrict__ chunks, const float* __restrict__ dsum, const float* __restrict__ A, float* __restrict__ state,
+    int row_len, const int* __restrict__ slot_ids, const int* __restrict__ seq_chunk, const int* __restrict__ q_start,
+    const TA* __restrict__ x_raw, int ldx, int C, int N, int K) {
+  const int i = blockIdx.x * SS_THREADS + threadIdx.x;
+  if (i >= C * N) return;
+  const int c = i / N, n = i % N;
+  const int b = blockIdx.y;
+  const float An = A[(size_t)c * N + n];
+  float* row = state + ((size_t)slot_ids[b] * C + c) * row_len;
+  float S = row[n];
+  for (int k = seq_chunk[b]; k < seq_chunk[b + 1]; ++k) {
+    float* at = chunks + ((size_t)k * C + c) * row_len + n;
+    const float add = *at;
+    *at = S;
+    S = expf(An * dsum[(size_t)k * C + c]) * S + add;
+  }
+  row[n] = S;
+  if (n == 0 && K > 1) {
+    float* tail = row + N;
+    const int t0 = q_start[b], L = q_start[b + 1] - t0, keep = K - 1;
+    float nt[SS_MAX_TAPS - 1];
+#pragma unroll
+    for (int j = 0; j < SS_MAX_TAPS - 1; ++j) {
+      if (j < keep) {
+        const int src = L - keep + j;
+        nt[j] = src >= 0 ? to_f<TA>(x_raw[(size_t)(t0 + src) * ldx + c]) : tail[j + L];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < SS_MAX_TAPS - 1; ++j)
+      if (j < keep) tail[j] = nt[j];
+  }
+}
+
+extern "C" int fg_scan_chunk_states(float* chunks, const float* dsum, const float* A, float* state, int row_len,
+                                    const int* slot_ids, const int* seq_chunk, const int* q_start, const void* x_raw,
+                                    int ldx, int n_seqs, int C, int N, int K, int act_dtype, hipStream_t stream) {
+  if (n_seqs <= 0) return FG_OK;
+  if (C <= 0 || N <= 0 || K < 1 || K > SS_MAX_TAPS || row_len < N + K - 1 || n_seqs > 65535 || (K > 1 && !x_raw) || !chunks ||
+      !dsum || !A || !state)
+    return FG_ERR_ARG;
+  dim3 grid((unsigned)(((long long)C * N + SS_THREADS - 1) / SS_THREADS), n_seqs);
+  if (act_dtype == FG_F32)
+    scan_chunk_states_kernel<float><<<grid, SS_THREADS, 0, stream>>>(chunks, dsum, A, state, row_len, slot_ids, seq_chunk,
+                                                                     q_start, (const float*)x_raw, ldx, C, N, K);
+  else if (act_dtype == FG_BF16)
+    scan_chunk_states_kernel<bf16_t><<<grid, SS_THREADS, 0, stream>>>(chunks, dsum, A, state, row_len, slot_ids, seq_chunk,
+                                                                      q_start, (const bf16_t*)x_raw, ldx, C, N, K);
+  else
+    return FG_ERR_ARG;
   return fg_launch_status();
 }

@@ -23,7 +23,7 @@
 #define SA_THREADS 256
 #define SA_WAVES 4
 #define SA_TILE 64
-#define SA_CHUNK_TILES 4
+#define SA_CHUNK_TILES 1
 #define SA_MAX_ITEMS 16  // (head, value dim) pairs a thread owns: heads * e <= 4096
 
 struct SigmoidAttentionArgs {

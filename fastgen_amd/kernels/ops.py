@@ -1414,7 +1414,12 @@ class _SelectiveArgs(ctypes.Structure):
                 ("ldz", ctypes.c_int), ("x_raw", ctypes.c_void_p), ("ldx", ctypes.c_int), ("state", ctypes.c_void_p),
                 ("row_len", ctypes.c_int), ("slot_ids", ctypes.c_void_p), ("q_start", ctypes.c_void_p),
                 ("out", ctypes.c_void_p), ("ldo", ctypes.c_int), ("C", ctypes.c_int), ("N", ctypes.c_int),
-                ("K", ctypes.c_int), ("LP", ctypes.c_int)]
+                ("K", ctypes.c_int), ("LP", ctypes.c_int), ("write_out", ctypes.c_int), ("write_state", ctypes.c_int),
+                ("write_tail", ctypes.c_int), ("dsum", ctypes.c_void_p)]
+
+
+SELECTIVE_CHUNK = 64  # tokens of a chunk where long runs of tokens are scanned chunk by chunk, side by side
+SELECTIVE_CHUNKED_FROM = 192  # the shortest run of tokens of one sequence for which a step is scanned so
 
 
 def _rows_of_width(t: torch.Tensor, T: int, width: int, name: str) -> None:
@@ -1454,7 +1459,7 @@ def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor
 def selective_scan(u: torch.Tensor, dt: torch.Tensor, dt_bias: Optional[torch.Tensor], A: torch.Tensor, bc: torch.Tensor,
                    b_col: int, c_col: int, D: Optional[torch.Tensor], z: Optional[torch.Tensor],
                    x_raw: Optional[torch.Tensor], taps: int, state: torch.Tensor, slot_ids: torch.Tensor,
-                   q_start: torch.Tensor, n_seqs: int, out: torch.Tensor) -> torch.Tensor:
+                   q_start: torch.Tensor, n_seqs: int, out: torch.Tensor, q_start_host=None) -> torch.Tensor:
     """The selective recurrence, token by token for every sequence of the step, in fp32:
     ``d = softplus(dt[t, c] + dt_bias[c])``; ``S[c, n] <- exp(d A[c, n]) S[c, n] + d u[t, c] B[t, n]``;
     ``out[t, c] = (sum_n S[c, n] C[t, n] + D[c] u[t, c]) * silu(z[t, c])``.
@@ -1463,7 +1468,12 @@ def selective_scan(u: torch.Tensor, dt: torch.Tensor, dt_bias: Optional[torch.Te
     fp32 ``[C, N]``; ``B[t, n] = bc[t, b_col + n]``, ``C[t, n] = bc[t, c_col + n]``; ``state`` fp32 ``[n_slots, C,
     row_len]`` holds ``S`` in its first ``N`` columns and, behind them, the last ``taps - 1`` rows of ``x_raw`` (the
     input of the convolution that made ``u``), which this call moves on by the step's tokens.  Sequence ``b`` has
-    the tokens ``q_start[b] .. q_start[b+1]-1`` and the state row ``slot_ids[b]``."""
+    the tokens ``q_start[b] .. q_start[b+1]-1`` and the state row ``slot_ids[b]``.
+
+    ``q_start_host``: ``q_start`` on the host.  With it, a step in which a sequence brings ``SELECTIVE_CHUNKED_FROM``
+    tokens or more is scanned in chunks of ``SELECTIVE_CHUNK`` tokens side by side (every chunk from a zero state,
+    then the states that the chunks start from, then every chunk from its start); the result differs from the
+    token-by-token scan's by rounding (a chunk's decay is the exponential of a sum, not a product)."""
     _gpu(u, dt, dt_bias, A, bc, D, z, x_raw, state, slot_ids, q_start, out)
     C, N = A.shape
     T = u.shape[0]
@@ -1501,8 +1511,33 @@ def selective_scan(u: torch.Tensor, dt: torch.Tensor, dt_bias: Optional[torch.Te
     a.bc, a.ldbc, a.b_col, a.c_col = bc.data_ptr(), bc.stride(0), int(b_col), int(c_col)
     a.state, a.row_len, a.slot_ids, a.q_start = state.data_ptr(), state.shape[2], slot_ids.data_ptr(), q_start.data_ptr()
     a.out, a.ldo, a.C, a.N, a.K, a.LP = out.data_ptr(), out.stride(0), C, N, int(taps), lanes
-    st = _lib.load("selective_scan").fg_selective_scan(ctypes.byref(a), int(n_seqs), _code(dt), _code(out), _stream(out))
-    _check(st, "selective_scan")
+    a.write_out = a.write_state = a.write_tail = 1
+    lib = _lib.load("selective_scan")
+    lens = np.diff(np.asarray(q_start_host[: n_seqs + 1])) if q_start_host is not None else None
+    if lens is None or not len(lens) or int(lens.max()) < SELECTIVE_CHUNKED_FROM or torch.cuda.is_current_stream_capturing():
+        _check(lib.fg_selective_scan(ctypes.byref(a), int(n_seqs), _code(dt), _code(out), _stream(out)), "selective_scan")
+        return out
+    # chunk by chunk: the chunks' first tokens, and which chunks each sequence has
+    starts, seq_chunk = [], [0]
+    for b in range(n_seqs):
+        starts.extend(range(int(q_start_host[b]), int(q_start_host[b + 1]), SELECTIVE_CHUNK))
+        seq_chunk.append(len(starts))
+    n_chunks = len(starts)
+    _need(n_chunks <= 65535 and n_seqs <= 65535, "too many chunks or sequences in one step")
+    plan = upload(np.asarray(starts + [int(q_start_host[n_seqs])] + seq_chunk + list(range(n_chunks)), dtype=np.int32),
+                  torch.int32, u.device)
+    chunk_start, seq_chunk_d, chunk_ids = plan[: n_chunks + 1], plan[n_chunks + 1 : n_chunks + n_seqs + 2], plan[n_chunks + n_seqs + 2 :]
+    row_len = state.shape[2]
+    chunks = torch.zeros((n_chunks, C, row_len), dtype=torch.float32, device=u.device)
+    dsum = torch.empty((n_chunks, C), dtype=torch.float32, device=u.device)
+    a.state, a.slot_ids, a.q_start, a.dsum = chunks.data_ptr(), chunk_ids.data_ptr(), chunk_start.data_ptr(), dsum.data_ptr()
+    a.write_out, a.write_state, a.write_tail = 0, 1, 0  # what every chunk adds to a zero state
+    _check(lib.fg_selective_scan(ctypes.byref(a), n_chunks, _code(dt), _code(out), _stream(out)), "selective_scan (chunks' sums)")
+    _check(lib.fg_scan_chunk_states(_ptr(chunks), _ptr(dsum), _ptr(A), _ptr(state), row_len, _ptr(slot_ids), _ptr(seq_chunk_d),
+                                    _ptr(q_start), _ptr(x_raw), x_raw.stride(0) if x_raw is not None else 0, int(n_seqs), C, N,
+                                    int(taps), _code(out), _stream(out)), "scan_chunk_states")
+    a.write_out, a.write_state, a.dsum = 1, 0, None  # every chunk from the state it starts from
+    _check(lib.fg_selective_scan(ctypes.byref(a), n_chunks, _code(dt), _code(out), _stream(out)), "selective_scan (chunks' outputs)")
     return out
 
 

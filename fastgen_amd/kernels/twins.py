@@ -618,9 +618,10 @@ def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor
 def selective_scan(u: torch.Tensor, dt: torch.Tensor, dt_bias: Optional[torch.Tensor], A: torch.Tensor, bc: torch.Tensor,
                    b_col: int, c_col: int, D: Optional[torch.Tensor], z: Optional[torch.Tensor],
                    x_raw: Optional[torch.Tensor], taps: int, state: torch.Tensor, slot_ids: torch.Tensor,
-                   q_start: torch.Tensor, n_seqs: int, out: torch.Tensor) -> torch.Tensor:
+                   q_start: torch.Tensor, n_seqs: int, out: torch.Tensor, q_start_host=None) -> torch.Tensor:
     """``S <- exp(d A) S + d u B``, ``y = S C + D u``, ``out = y * silu(z)`` token by token, ``d = softplus(dt + dt_bias)``; the
-    state's rows hold ``S`` and behind it the convolution's last ``taps - 1`` inputs, moved on by this step."""
+    state's rows hold ``S`` and behind it the convolution's last ``taps - 1`` inputs, moved on by this step.
+    (``q_start_host`` only lets the kernels cut long runs of tokens into chunks.)"""
     C, N = A.shape
     for b in range(n_seqs):
         t0, t1 = int(q_start[b]), int(q_start[b + 1])

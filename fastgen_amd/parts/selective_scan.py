@@ -91,7 +91,8 @@ class SelectiveScan(Mixer):
         dt = linear(narrow, self.w_dt, out_dtype=torch.float32)
         y = torch.empty((T, C), dtype=x.dtype, device=x.device)
         ops.selective_scan(u, dt, self.dt_bias, self.A, narrow, R, R + N, self.D, rows[:, C:], rows, self.taps,
-                           store.state, ctx.slot_ids, ctx.q_start, ctx.n_seqs, y)
+                           store.state, ctx.slot_ids, ctx.q_start, ctx.n_seqs, y,
+                           q_start_host=None if ctx.graph_capacity else ctx.q_start_host)
         return linear(y, self.wo, partials_ok=True)
 
 

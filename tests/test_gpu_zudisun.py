@@ -110,7 +110,8 @@ def test_grouped_sigmoid_router_kernel(dtype, T, E, top, groups, keep):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("C,N,R,K,lens", [(10, 4, 3, 3, [5, 1, 8]), (70, 1, 1, 1, [4, 2]), (36, 37, 2, 9, [2, 1, 1, 30]),
-                                          (256, 24, 10, 4, [130, 1, 1, 17]), (24, 300, 8, 2, [9, 3]), (8, 600, 8, 16, [20])])
+                                          (256, 24, 10, 4, [130, 1, 1, 17]), (24, 300, 8, 2, [9, 3]), (8, 600, 8, 16, [20]),
+                                          (48, 16, 4, 4, [300, 1, 70, 200]), (20, 5, 2, 3, [192])])
 def test_convolution_and_scan_kernels_carry_their_state(dtype, C, N, R, K, lens):
     """Two steps of every sequence, through slots in another order: the kernels against their twins, the state
     and the convolution's tail after each step too."""
@@ -140,7 +141,7 @@ def test_convolution_and_scan_kernels_carry_their_state(dtype, C, N, R, K, lens)
         _close(ug, u, dtype, f"convolution, step {step}")
         # the scan from the twin's convolution, so that its own error alone is measured
         ops.selective_scan(u.to(DEV), dt.to(DEV), db.to(DEV), A.to(DEV), bc.to(DEV), R, R + N, D.to(DEV), rows_g[:, C:], rows_g, K,
-                           state_g, slots.to(DEV), q_start.to(DEV), B, og)
+                           state_g, slots.to(DEV), q_start.to(DEV), B, og, q_start_host=q_start.numpy())  # (long runs in chunks)
         _close(og, out, dtype, f"scan, step {step}")
         tol = 2e-5 if dtype == torch.float32 else 2e-3
         torch.testing.assert_close(state_g.cpu(), state, rtol=tol, atol=tol)
