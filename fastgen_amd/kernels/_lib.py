@@ -56,6 +56,7 @@ LIBRARIES: Dict[str, str] = {
 VARIANT_LIBRARIES: Dict[str, tuple] = {
     "attention_mfma": ("attention_mfma.hip", "FG_HD", tuple(range(16, 257, 16)), ()),
     "attention_mfma_exact": ("attention_mfma.hip", "FG_HD", tuple(range(16, 257, 16)), ("-DFG_EXACT_P=1",)),
+    "sigmoid_attention_mfma": ("sigmoid_attention_mfma.hip", "FG_HD", tuple(range(16, 257, 16)), ()),
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

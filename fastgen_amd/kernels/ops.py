@@ -1559,12 +1559,105 @@ def sigmoid_attention_chunk_keys() -> int:
     return int(_lib.load("sigmoid_attention").fg_sigmoid_attention_chunk_keys())
 
 
+class _SigmoidTileArgs(ctypes.Structure):
+    _fields_ = [("q", ctypes.c_void_p), ("q_stride", ctypes.c_int), ("q_hs", ctypes.c_int), ("k_pages", ctypes.c_void_p),
+                ("v_pages", ctypes.c_void_p), ("block_table", ctypes.c_void_p), ("bt_stride", ctypes.c_int),
+                ("items", ctypes.c_void_p), ("n_items", ctypes.c_int), ("positions", ctypes.c_void_p),
+                ("n_tokens", ctypes.c_int), ("n_heads", ctypes.c_int), ("n_kv", ctypes.c_int), ("d", ctypes.c_int),
+                ("e", ctypes.c_int), ("page_size", ctypes.c_int), ("talk", ctypes.c_void_p), ("mixed", ctypes.c_void_p),
+                ("n_dist", ctypes.c_int), ("gate", ctypes.c_void_p), ("gate_stride", ctypes.c_int), ("out", ctypes.c_void_p),
+                ("out_stride", ctypes.c_int), ("partial", ctypes.c_void_p), ("n_chunks", ctypes.c_int),
+                ("chunk_keys", ctypes.c_int)]
+
+
+SIGMOID_TILE_TOKENS = 16  # query tokens of an item of the matrix-core kernel
+SIGMOID_TILE_HEADS = 16  # the most heads it mixes
+SIGMOID_TILE_CHUNK = 512  # keys of a chunk, at least; at most SIGMOID_TILE_MAX_CHUNKS chunks
+SIGMOID_TILE_MAX_CHUNKS = 8
+
+
+def sigmoid_attention_items(q_lens, q_start, n_cached) -> np.ndarray:
+    """The step's sequences cut into items of up to 16 consecutive tokens: int32 ``[n, 4]`` of (sequence, first flat
+    token, tokens, position of the first token), those with the most keys first."""
+    items = [(b, int(q_start[b]) + i, min(SIGMOID_TILE_TOKENS, int(n) - i), int(n_cached[b]) + i)
+             for b, n in enumerate(q_lens) for i in range(0, int(n), SIGMOID_TILE_TOKENS)]
+    items.sort(key=lambda it: -(it[3] + it[2]))
+    return np.asarray(items, dtype=np.int32).reshape(-1, 4)
+
+
+def sigmoid_attention_mixed(scale: float, n_heads: int, dist_bias: Optional[torch.Tensor], talk: Optional[torch.Tensor],
+                            head_bias: Optional[torch.Tensor], device):
+    """What the matrix-core kernel takes in place of the table, the matrix and the biases (None with more than 16
+    heads): the mixing matrix (or the identity) times the scale, zero padded to ``[16, 16]``, and ``[n_dist, 16]``:
+    the distance table mixed over the heads by the same matrix plus the heads' biases (mixing is linear, so the
+    bias can be mixed apart from the products and once for all steps).  fp32."""
+    H = int(n_heads)
+    if H > SIGMOID_TILE_HEADS:
+        return None
+    T = talk.float() if talk is not None else torch.eye(H, device=device)
+    wide = torch.zeros((SIGMOID_TILE_HEADS, SIGMOID_TILE_HEADS), dtype=torch.float32, device=device)
+    wide[:H, :H] = T * float(scale)
+    rel = dist_bias.float() if dist_bias is not None else torch.zeros((1, H), device=device)
+    m = rel @ T.T
+    if head_bias is not None:
+        m = m + head_bias.float()
+    table = torch.zeros((m.shape[0], SIGMOID_TILE_HEADS), dtype=torch.float32, device=device)
+    table[:, :H] = m
+    return wide.contiguous(), table.contiguous()
+
+
+def _sigmoid_attention_tiles(q, head_dim, out, v_head_dim, k_pages, v_pages, block_table, positions, n_heads, gate, max_keys,
+                             items, mixed) -> torch.Tensor:
+    T, H, d, e = q.shape[0], int(n_heads), int(head_dim), int(v_head_dim)
+    _need(mixed is not None and len(mixed) == 2, "the matrix-core kernel takes sigmoid_attention_mixed's pair")
+    talk, table = mixed
+    _gpu(talk, table)
+    _need(k_pages.dim() == 4 and k_pages.is_contiguous() and k_pages.dtype == torch.bfloat16, "k_pages must be contiguous bfloat16 [n_pages, G, P, hd]")
+    n_pages, G, P, hd = k_pages.shape
+    _need(v_pages.is_contiguous() and v_pages.shape == (n_pages, G, hd, P) and v_pages.dtype == torch.bfloat16,
+          "v_pages must be contiguous bfloat16 [n_pages, G, hd, P]")
+    _need(0 < H <= SIGMOID_TILE_HEADS and H % G == 0 and 0 < d <= hd and 0 < e <= hd and hd % 16 == 0 and hd <= 256 and P % 32 == 0,
+          "at most 16 heads, head sizes at most the cache's (a multiple of 16 up to 256), pages of a multiple of 32 keys")
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "q and out must be bfloat16")
+    _rows_of_width(q, T, H * d, "q")
+    _rows_of_width(out, T, H * e, "out")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "block_table must be int32 [B, pages]")
+    _i32(positions, "positions", T)
+    _i32(items, "items")
+    _need(items.dim() == 2 and items.shape[1] == 4 and items.is_contiguous() and items.data_ptr() % 16 == 0, "items must be [n, 4], 16-byte aligned")
+    _need(talk.dtype == torch.float32 and talk.is_contiguous() and talk.shape == (SIGMOID_TILE_HEADS, SIGMOID_TILE_HEADS)
+          and table.dtype == torch.float32 and table.is_contiguous() and table.dim() == 2 and table.shape[1] == SIGMOID_TILE_HEADS
+          and table.data_ptr() % 16 == 0, "mixed must be sigmoid_attention_mixed's pair")
+    a = _SigmoidTileArgs()
+    if gate is not None:
+        _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] == T
+              and gate.shape[1] >= H, "gate must be float32 [T, >= H]")
+        a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
+    max_keys = max(int(max_keys), 1)
+    chunk = max(SIGMOID_TILE_CHUNK, -(-max_keys // (SIGMOID_TILE_MAX_CHUNKS * 32)) * 32)
+    n_chunks = -(-max_keys // chunk)
+    partial = None
+    if n_chunks > 1:
+        partial = torch.empty((n_chunks, T, H * e), dtype=torch.float32, device=q.device)
+        a.partial = partial.data_ptr()
+    a.n_chunks, a.chunk_keys = n_chunks, chunk
+    a.q, a.q_stride, a.q_hs = q.data_ptr(), q.stride(0), d
+    a.k_pages, a.v_pages, a.block_table, a.bt_stride = k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.stride(0)
+    a.items, a.n_items, a.positions, a.n_tokens = items.data_ptr(), items.shape[0], positions.data_ptr(), T
+    a.n_heads, a.n_kv, a.d, a.e, a.page_size = H, G, d, e, P
+    a.talk, a.mixed, a.n_dist = talk.data_ptr(), table.data_ptr(), table.shape[0]
+    a.out, a.out_stride = out.data_ptr(), out.stride(0)
+    st = _lib.load(f"sigmoid_attention_mfma@{hd}").fg_sigmoid_attention_tiles(ctypes.byref(a), _stream(q))
+    _check(st, "sigmoid_attention (matrix cores)")
+    return out
+
+
 def sigmoid_attention(q: torch.Tensor, head_dim: int, out: torch.Tensor, v_head_dim: int, k_pages: torch.Tensor,
                       v_pages: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
                       positions: torch.Tensor, n_heads: int, scale: float,
                       dist_bias: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None,
                       head_bias: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
-                      split_for: int = 0) -> torch.Tensor:
+                      split_for: int = 0, items: Optional[torch.Tensor] = None, mixed=None) -> torch.Tensor:
     """Causal attention over the paged cache whose weights are sigmoids and are not normalised over the keys.
 
     For the query at flat row ``t`` (position ``p`` of sequence ``seq_of_token[t]``) and every key ``j <= p`` of its
@@ -1575,8 +1668,16 @@ def sigmoid_attention(q: torch.Tensor, head_dim: int, out: torch.Tensor, v_head_
     the cache's dtype; keys and values are read from ``k_pages [n_pages, G, P, hd]`` and ``v_pages [n_pages, G, hd,
     P]`` (their first ``head_dim`` and ``v_head_dim`` elements).  ``split_for`` > 0: the keys of every token are
     cut over several workgroups, enough for sequences of that many keys (for few tokens with many keys); the
-    result has the same bits either way."""
-    _gpu(q, out, k_pages, v_pages, block_table, seq_of_token, positions, dist_bias, talk, head_bias, gate)
+    result has the same bits either way.
+
+    ``items`` (device int32 ``[n, 4]`` from :func:`sigmoid_attention_items`, covering every token of the step) and
+    ``mixed`` (:func:`sigmoid_attention_mixed` of the same scale, table, matrix and biases): bfloat16 prompt portions
+    on the matrix cores, an item a workgroup (``split_for``: the most keys a sequence has); the result differs from
+    the general kernel's by rounding."""
+    _gpu(q, out, k_pages, v_pages, block_table, seq_of_token, positions, dist_bias, talk, head_bias, gate, items)
+    if items is not None:
+        return _sigmoid_attention_tiles(q, head_dim, out, v_head_dim, k_pages, v_pages, block_table, positions, n_heads, gate,
+                                        split_for, items, mixed)
     T, H, d, e = q.shape[0], int(n_heads), int(head_dim), int(v_head_dim)
     _need(k_pages.dim() == 4 and k_pages.is_contiguous(), "k_pages must be contiguous [n_pages, G, P, hd]")
     n_pages, G, P, hd = k_pages.shape

@@ -649,10 +649,11 @@ def sigmoid_attention(q: torch.Tensor, head_dim: int, out: torch.Tensor, v_head_
                       positions: torch.Tensor, n_heads: int, scale: float,
                       dist_bias: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None,
                       head_bias: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
-                      split_for: int = 0) -> torch.Tensor:
+                      split_for: int = 0, items: Optional[torch.Tensor] = None, mixed=None) -> torch.Tensor:
     """Token ``t`` at position ``p`` of sequence ``b`` over the keys ``0..p`` of its sequence: scores ``q . k * scale``
     plus ``dist_bias[min(p - j, n_dist - 1), h]``, mixed over the heads by ``talk``, plus ``head_bias``; weights
-    ``sigmoid(score)``, not normalised; the heads' sums of weighted values times ``sigmoid(gate)``."""
+    ``sigmoid(score)``, not normalised; the heads' sums of weighted values times ``sigmoid(gate)``.  (``split_for``,
+    ``items`` and ``mixed`` only choose how the kernels cut the work.)"""
     H, d, e = n_heads, head_dim, v_head_dim
     n_kv = k_pages.shape[1]
     rep = H // n_kv

@@ -66,6 +66,7 @@ class SigmoidAttention(Mixer):
         self.w_in: Optional[StreamedMatrix] = None
         self.wo: Optional[StreamedMatrix] = None
         self.rel = self.talk = self.pb = None
+        self.mixed = None  # what the matrix-core kernel takes in place of the table, the matrix and the biases
         self.blend = 0.0
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -103,6 +104,7 @@ class SigmoidAttention(Mixer):
             self.pb = f32("head_bias")
         if self.value_mix:
             self.blend = float(t("value_mix").float())
+        self.mixed = ops.sigmoid_attention_mixed(self.scale, self.n_heads, self.rel, self.talk, self.pb, device)
 
     def paged_need(self) -> PagedNeed:
         return PagedNeed(self.n_kv_heads, self.cache_dim)
@@ -127,12 +129,24 @@ class SigmoidAttention(Mixer):
             positions=ctx.positions, q_temp_coef=self.q_temp_coef, q_temp_every=self.q_temp_every,
             v_first=v_first, v_blend=self.blend)
         out = torch.empty((T, H * e), dtype=x.dtype, device=x.device)
-        split_for = 0
+        split_for, items = 0, None
         if T <= SPLIT_MAX_TOKENS:
             split_for = ctx.graph_capacity or ctx.max_kv_len
+        elif (self.mixed is not None and x.dtype == torch.bfloat16 and not ctx.graph_capacity
+              and store.k_pages.shape[2] % 32 == 0 and self.cache_dim <= 256):
+            # prompt portions in bfloat16: the matrix cores, an item of up to 16 tokens a workgroup (if the step is
+            # not mostly single tokens, which would each be an item)
+            items = ctx.scratch.get("sigmoid_items")
+            if items is None:
+                host = ops.sigmoid_attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached)
+                items = ctx.scratch["sigmoid_items"] = ops.upload(host, torch.int32, x.device) if 4 * len(host) <= T else False
+            if items is False:
+                items = None
+            else:
+                split_for = ctx.max_kv_len
         ops.sigmoid_attention(q, d, out, e, store.k_pages, store.v_pages, group.block_table, ctx.seq_of_token,
                               ctx.positions, H, self.scale, self.rel, self.talk, self.pb,
-                              rows[:, g_col:] if self.head_gate else None, split_for=split_for)
+                              rows[:, g_col:] if self.head_gate else None, split_for=split_for, items=items, mixed=self.mixed)
         return linear(out, self.wo, partials_ok=True)
 
 

@@ -163,7 +163,8 @@ def _paged(T, n_kv, hc, P, dtype, seed):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,e,hc,P,rows,far,every,T", [(4, 2, 6, 4, 8, 8, 6, 9.0, 3, 29), (8, 4, 80, 48, 80, 64, 24, 150.0, 100, 700),
                                                             (3, 3, 8, 10, 16, 16, 8, 40.0, 1, 150), (34, 2, 8, 8, 16, 16, 64, 33.0, 7, 90),
-                                                            (5, 1, 20, 48, 48, 32, 9, 1000.0, 1000, 300)])
+                                                            (5, 1, 20, 48, 48, 32, 9, 1000.0, 1000, 300),
+                                                            (16, 4, 64, 64, 64, 64, 16, 600.0, 50, 1100), (12, 3, 32, 16, 32, 32, 10, 64.0, 9, 130)])
 def test_prepare_and_sigmoid_attention_kernels(dtype, H, G, d, e, hc, P, rows, far, every, T):
     """Unit norms per head, the query's temperature, blended values, pages; then the attention over the pages for
     a whole prompt, for its last tokens alone with the keys cut over workgroups, and both with the same bits."""
@@ -206,6 +207,26 @@ def test_prepare_and_sigmoid_attention_kernels(dtype, H, G, d, e, hc, P, rows, f
     ops.sigmoid_attention(q[last].to(DEV), d, cut, e, *args, seq[last].to(DEV), pos[last].to(DEV), *rest,
                           gate[last].contiguous().to(DEV), split_for=T)
     assert torch.equal(cut, og[last]), "keys cut over workgroups: the same bits"
+    if dtype == torch.bfloat16 and P % 32 == 0 and H <= ops.SIGMOID_TILE_HEADS:
+        # prompt portions on the matrix cores: the whole prompt, and its last 40 tokens behind the cached rest
+        mixed = ops.sigmoid_attention_mixed(0.4, H, spread.to(DEV), talk.to(DEV), pb.to(DEV), DEV)
+        items = ops.upload(ops.sigmoid_attention_items([0, T], [0, 0, T], [0, 0]), torch.int32, DEV)
+        assert int(items[:, 2].sum()) == T and int(items[:, 2].max()) <= 16
+        tiles = torch.empty(T, H * e, dtype=dtype, device=DEV)
+        ops.sigmoid_attention(q.to(DEV), d, tiles, e, *args, seq.to(DEV), pos.to(DEV), *rest, gate.to(DEV), split_for=T,
+                              items=items, mixed=mixed)
+        torch.testing.assert_close(tiles.float().cpu(), out.float(), **tol)
+        part = slice(T - 40, T)
+        items = ops.upload(ops.sigmoid_attention_items([0, 40], [0, 0, 40], [0, T - 40]), torch.int32, DEV)
+        tiles = torch.empty(40, H * e, dtype=dtype, device=DEV)
+        ops.sigmoid_attention(q[part].to(DEV), d, tiles, e, *args, seq[part].to(DEV), pos[part].to(DEV), *rest,
+                              gate[part].contiguous().to(DEV), split_for=T, items=items, mixed=mixed)
+        torch.testing.assert_close(tiles.float().cpu(), out[part].float(), **tol)
+        plain = ops.sigmoid_attention_mixed(0.4, H, None, None, pb.to(DEV), DEV)
+        twins.sigmoid_attention(q[part], d, out[part], e, kp, vp, table, seq[part], pos[part], H, 0.4, None, None, pb, None)
+        ops.sigmoid_attention(q[part].to(DEV), d, tiles, e, *args, seq[part].to(DEV), pos[part].to(DEV), H, 0.4, None, None,
+                              pb.to(DEV), None, split_for=T, items=items, mixed=plain)
+        torch.testing.assert_close(tiles.float().cpu(), out[part].float(), **tol)
     # without the optional parts
     twins.sigmoid_attention(q, d, out, e, kp, vp, table, seq, pos, H, 0.4, None, None, pb, None)
     ops.sigmoid_attention(q.to(DEV), d, og, e, *args, seq.to(DEV), pos.to(DEV), H, 0.4, None, None, pb.to(DEV), None)
@@ -264,9 +285,11 @@ def test_float32_every_cut_batch_and_reuse(cases, exact, name):
 def test_bfloat16_every_cut_batch_and_reuse(cases, name):
     config, weights, folder, toks, want = cases[name]
     noise = {r: plain_zudisun_forward(config, weights, t, torch.bfloat16) for r, t in toks.items()}
-    runner = make_runner(folder, torch.bfloat16, page_size=16, max_tokens=304, max_requests=4)
-    for kind, tr in _all_traces(LENGTHS).items():
-        _close_to_plain(run_trace(runner, tr, toks), want, noise, torch.bfloat16, f"zudisun {name} {kind} bfloat16", _routed(config))
+    for page, pool in ((16, 304), (64, 768)):  # (pages of 64: prompt portions of the attention run on the matrix cores)
+        runner = make_runner(folder, torch.bfloat16, page_size=page, max_tokens=pool, max_requests=4)
+        for kind, tr in _all_traces(LENGTHS).items():
+            _close_to_plain(run_trace(runner, tr, toks), want, noise, torch.bfloat16, f"zudisun {name} {kind} bfloat16, pages of {page}",
+                            _routed(config))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -329,8 +352,8 @@ def test_long_prompts_beside_short_ones(cases, name):
     exact = {r: plain_zudisun_forward(config, weights, t, torch.float64) for r, t in toks.items()}
     noise = {r: plain_zudisun_forward(config, weights, t, torch.bfloat16) for r, t in toks.items()}
     together = [([("p", 0, 700), ("q", 0, 260), ("r", 0, 3)], ["p", "q", "r"])]
-    for dtype in (torch.float32, torch.bfloat16):
-        runner = make_runner(folder, dtype, page_size=16, max_tokens=1024, max_requests=3)
+    for dtype, page in ((torch.float32, 16), (torch.bfloat16, 16), (torch.bfloat16, 64)):
+        runner = make_runner(folder, dtype, page_size=page, max_tokens=1152, max_requests=3)
         for kind, tr in (("whole", traces.whole(lengths)), ("together", together),
                          ("halves", traces.chunks(lengths, sizes=(390, 310))), ("portions", traces.chunks(lengths))):
             got = run_trace(runner, tr, toks)
@@ -396,8 +419,8 @@ def test_keys_at_the_edges_of_the_distance_table(tmp_path):
         if row >= 9:
             assert float(moved[lo + 5 :].min()) > 0.02 * float(want["s"].abs().max()), "the table's steps do not decide"
         folder = save_model_folder(tmp_path / f"r{row}_{int(far)}", config, w)
-        for dtype in (torch.float32, torch.bfloat16):
-            runner = make_runner(folder, dtype, page_size=16, max_tokens=240, max_requests=1)
+        for dtype, page in ((torch.float32, 16), (torch.bfloat16, 16), (torch.bfloat16, 64)):
+            runner = make_runner(folder, dtype, page_size=page, max_tokens=256, max_requests=1)
             noise = {"s": plain_zudisun_forward(config, w, toks["s"], torch.bfloat16)} if dtype == torch.bfloat16 else None
             for tr in (traces.whole({"s": n}), traces.tail({"s": n}, 170), traces.chunks({"s": n}),
                        traces.chunks({"s": n}, sizes=(2, 3, 2, 5))):
