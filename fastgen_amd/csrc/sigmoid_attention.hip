@@ -181,18 +181,25 @@ __global__ __launch_bounds__(SA_THREADS) void sigmoid_attention_kernel(const Sig
   }
 }
 
-// out[t, item] = (sum over the token's chunks, in order) * sigmoid(gate[t, head])
+// out[t, item] = (sum over the token's chunks, in order) * sigmoid(gate[t, head]); a thread an element
 template <class T>
 __global__ __launch_bounds__(SA_THREADS) void sigmoid_attention_combine_kernel(const SigmoidAttentionArgs a) {
   const int t = blockIdx.x;
   const int n_items = a.n_heads * a.e;
+  const int item = blockIdx.y * SA_THREADS + threadIdx.x;
+  if (item >= n_items) return;
   const int last_chunk = a.positions[t] / (SA_CHUNK_TILES * SA_TILE);
-  for (int item = threadIdx.x; item < n_items; item += SA_THREADS) {
-    float y = 0.f;
-    for (int c = 0; c <= last_chunk; ++c) y += a.partial[((size_t)c * a.n_tokens + t) * n_items + item];
-    if (a.gate) y *= 1.f / (1.f + expf(-a.gate[(size_t)t * a.gate_stride + item / a.e]));
-    ((T*)a.out)[(size_t)t * a.out_stride + item] = from_f<T>(y);
+  const size_t step = (size_t)a.n_tokens * n_items;
+  const float* p = a.partial + (size_t)t * n_items + item;
+  float y = 0.f;
+  int c = 0;
+  for (; c + 4 <= last_chunk + 1; c += 4) {  // four loads in flight, added in order
+    const float p0 = p[c * step], p1 = p[(c + 1) * step], p2 = p[(c + 2) * step], p3 = p[(c + 3) * step];
+    y += p0; y += p1; y += p2; y += p3;
   }
+  for (; c <= last_chunk; ++c) y += p[c * step];
+  if (a.gate) y *= 1.f / (1.f + expf(-a.gate[(size_t)t * a.gate_stride + item / a.e]));
+  ((T*)a.out)[(size_t)t * a.out_stride + item] = from_f<T>(y);
 }
 
 extern "C" int fg_sigmoid_attention_chunk_keys() { return SA_CHUNK_TILES * SA_TILE; }
@@ -209,12 +216,13 @@ extern "C" int fg_sigmoid_attention(const SigmoidAttentionArgs* args, int dtype,
   if (lds > 65536) return FG_ERR_ARG;
   dim3 grid(a.n_tokens, a.partial ? a.n_chunks : 1);
   if (grid.y > 65535) return FG_ERR_ARG;
+  const dim3 combine_grid(a.n_tokens, (a.n_heads * a.e + SA_THREADS - 1) / SA_THREADS);
   if (dtype == FG_F32) {
     sigmoid_attention_kernel<float><<<grid, SA_THREADS, lds, stream>>>(a);
-    if (a.partial) sigmoid_attention_combine_kernel<float><<<a.n_tokens, SA_THREADS, 0, stream>>>(a);
+    if (a.partial) sigmoid_attention_combine_kernel<float><<<combine_grid, SA_THREADS, 0, stream>>>(a);
   } else if (dtype == FG_BF16) {
     sigmoid_attention_kernel<bf16_t><<<grid, SA_THREADS, lds, stream>>>(a);
-    if (a.partial) sigmoid_attention_combine_kernel<bf16_t><<<a.n_tokens, SA_THREADS, 0, stream>>>(a);
+    if (a.partial) sigmoid_attention_combine_kernel<bf16_t><<<combine_grid, SA_THREADS, 0, stream>>>(a);
   } else {
     return FG_ERR_ARG;
   }

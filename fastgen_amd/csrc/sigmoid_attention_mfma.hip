@@ -218,17 +218,24 @@ __global__ __launch_bounds__(ST_THREADS) void sigmoid_tile_kernel(const SigmoidT
   }
 }
 
-// out[t, x] = (sum over the token's chunks, in order) * sigmoid(gate[t, head])
+// out[t, x] = (sum over the token's chunks, in order) * sigmoid(gate[t, head]); a thread an element
 __global__ __launch_bounds__(ST_THREADS) void sigmoid_tile_combine_kernel(const SigmoidTileArgs a) {
   const int t = blockIdx.x;
   const int n_items = a.n_heads * a.e;
+  const int x = blockIdx.y * ST_THREADS + threadIdx.x;
+  if (x >= n_items) return;
   const int last_chunk = a.positions[t] / a.chunk_keys;
-  for (int x = threadIdx.x; x < n_items; x += ST_THREADS) {
-    float y = 0.f;
-    for (int c = 0; c <= last_chunk; ++c) y += a.partial[((size_t)c * a.n_tokens + t) * n_items + x];
-    if (a.gate) y *= 1.f / (1.f + expf(-a.gate[(size_t)t * a.gate_stride + x / a.e]));
-    a.out[(size_t)t * a.out_stride + x] = from_f<bf16_t>(y);
+  const size_t step = (size_t)a.n_tokens * n_items;
+  const float* p = a.partial + (size_t)t * n_items + x;
+  float y = 0.f;
+  int c = 0;
+  for (; c + 4 <= last_chunk + 1; c += 4) {  // four loads in flight, added in order
+    const float p0 = p[c * step], p1 = p[(c + 1) * step], p2 = p[(c + 2) * step], p3 = p[(c + 3) * step];
+    y += p0; y += p1; y += p2; y += p3;
   }
+  for (; c <= last_chunk; ++c) y += p[c * step];
+  if (a.gate) y *= 1.f / (1.f + expf(-a.gate[(size_t)t * a.gate_stride + x / a.e]));
+  a.out[(size_t)t * a.out_stride + x] = from_f<bf16_t>(y);
 }
 
 extern "C" int fg_sigmoid_tile_head_dim() { return HD; }
@@ -254,6 +261,7 @@ extern "C" int fg_sigmoid_attention_tiles(const SigmoidTileArgs* args, hipStream
   else if (hpw == 2) GO(2);
   else GO(4);
 #undef GO
-  if (a.partial) sigmoid_tile_combine_kernel<<<a.n_tokens, ST_THREADS, 0, stream>>>(a);
+  if (a.partial)
+    sigmoid_tile_combine_kernel<<<dim3(a.n_tokens, (a.n_heads * a.e + ST_THREADS - 1) / ST_THREADS), ST_THREADS, 0, stream>>>(a);
   return fg_launch_status();
 }

@@ -1574,6 +1574,8 @@ SIGMOID_TILE_TOKENS = 16  # query tokens of an item of the matrix-core kernel
 SIGMOID_TILE_HEADS = 16  # the most heads it mixes
 SIGMOID_TILE_CHUNK = 512  # keys of a chunk, at least; at most SIGMOID_TILE_MAX_CHUNKS chunks
 SIGMOID_TILE_MAX_CHUNKS = 8
+SIGMOID_TILE_FEW_TOKENS = 64  # up to so many tokens a step, chunks of SIGMOID_TILE_FEW_CHUNK keys, as many as it takes
+SIGMOID_TILE_FEW_CHUNK = 128
 
 
 def sigmoid_attention_items(q_lens, q_start, n_cached) -> np.ndarray:
@@ -1634,7 +1636,10 @@ def _sigmoid_attention_tiles(q, head_dim, out, v_head_dim, k_pages, v_pages, blo
               and gate.shape[1] >= H, "gate must be float32 [T, >= H]")
         a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
     max_keys = max(int(max_keys), 1)
-    chunk = max(SIGMOID_TILE_CHUNK, -(-max_keys // (SIGMOID_TILE_MAX_CHUNKS * 32)) * 32)
+    if T <= SIGMOID_TILE_FEW_TOKENS:  # decoding: many small chunks, so that few tokens fill the device
+        chunk = SIGMOID_TILE_FEW_CHUNK
+    else:
+        chunk = max(SIGMOID_TILE_CHUNK, -(-max_keys // (SIGMOID_TILE_MAX_CHUNKS * 32)) * 32)
     n_chunks = -(-max_keys // chunk)
     partial = None
     if n_chunks > 1:

@@ -130,12 +130,18 @@ class SigmoidAttention(Mixer):
             v_first=v_first, v_blend=self.blend)
         out = torch.empty((T, H * e), dtype=x.dtype, device=x.device)
         split_for, items = 0, None
-        if T <= SPLIT_MAX_TOKENS:
+        # bfloat16 with pages of a multiple of 32 keys and at most 16 heads: the matrix cores, an item of up to 16
+        # tokens of a sequence a workgroup
+        tiles_ok = (self.mixed is not None and x.dtype == torch.bfloat16 and store.k_pages.shape[2] % 32 == 0
+                    and self.cache_dim <= 256)
+        if tiles_ok and ctx.seq_records is not None and int(ctx.q_lens.max()) <= ops.SIGMOID_TILE_TOKENS:
+            # every sequence is one item: its records are in the step's buffer already (and are refreshed with it
+            # when the step is a replayed graph)
+            items, split_for = ctx.seq_records, ctx.graph_capacity or ctx.max_kv_len
+        elif T <= SPLIT_MAX_TOKENS:
             split_for = ctx.graph_capacity or ctx.max_kv_len
-        elif (self.mixed is not None and x.dtype == torch.bfloat16 and not ctx.graph_capacity
-              and store.k_pages.shape[2] % 32 == 0 and self.cache_dim <= 256):
-            # prompt portions in bfloat16: the matrix cores, an item of up to 16 tokens a workgroup (if the step is
-            # not mostly single tokens, which would each be an item)
+        elif tiles_ok and not ctx.graph_capacity:
+            # prompt portions (if the step is not mostly single tokens, which would each be an item)
             items = ctx.scratch.get("sigmoid_items")
             if items is None:
                 host = ops.sigmoid_attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached)

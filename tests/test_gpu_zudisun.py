@@ -222,6 +222,11 @@ def test_prepare_and_sigmoid_attention_kernels(dtype, H, G, d, e, hc, P, rows, f
         ops.sigmoid_attention(q[part].to(DEV), d, tiles, e, *args, seq[part].to(DEV), pos[part].to(DEV), *rest,
                               gate[part].contiguous().to(DEV), split_for=T, items=items, mixed=mixed)
         torch.testing.assert_close(tiles.float().cpu(), out[part].float(), **tol)
+        # single tokens of three sequences (here: three positions of one), the keys in many small chunks
+        singles = ops.upload([[1, 0, 1, T - 3], [1, 1, 1, T - 2], [1, 2, 1, T - 1]], torch.int32, DEV)
+        ops.sigmoid_attention(q[last].to(DEV), d, cut, e, *args, seq[last].to(DEV), pos[last].to(DEV), *rest,
+                              gate[last].contiguous().to(DEV), split_for=T + 200, items=singles, mixed=mixed)
+        torch.testing.assert_close(cut.float().cpu(), out[last].float(), **tol)
         plain = ops.sigmoid_attention_mixed(0.4, H, None, None, pb.to(DEV), DEV)
         twins.sigmoid_attention(q[part], d, out[part], e, kp, vp, table, seq[part], pos[part], H, 0.4, None, None, pb, None)
         ops.sigmoid_attention(q[part].to(DEV), d, tiles, e, *args, seq[part].to(DEV), pos[part].to(DEV), H, 0.4, None, None,
