@@ -548,18 +548,18 @@ def _zudisun_kernels(z: dict, rows: int, context: int) -> dict:
     kv_bytes = (n_seqs * per_seq * 2 * G * d + 2 * rows * H * d) * 2
     # per (query, key) pair: the two products (matrix cores), and in fp32 by design: the heads' mixing (2 H^2), the
     # bias, scale and sigmoid (about 8 a head)
-    tiles = {}
-    if not decode:  # prompt portions run on the matrix cores, an item of 16 tokens a workgroup
-        tiles = dict(items=ops.upload(ops.sigmoid_attention_items([rows], [0, rows], [0]), torch.int32, "cuda"),
-                     mixed=ops.sigmoid_attention_mixed(d ** -0.5, H, rel, talk, pb, "cuda"))
-        split = rows
+    # bfloat16 runs on the matrix cores, an item of up to 16 tokens of a sequence a workgroup and chunk of keys
+    if decode:
+        items = [[b, b, 1, context - 1] for b in range(rows)]
+    else:
+        items, split = ops.sigmoid_attention_items([rows], [0, rows], [0]), rows
+    tiles = dict(items=ops.upload(items, torch.int32, "cuda"), mixed=ops.sigmoid_attention_mixed(d ** -0.5, H, rel, talk, pb, "cuda"))
     put("sigmoid_attention", lambda: ops.sigmoid_attention(q, d, o, d, kp, vp, table, seq_of_token, positions, H, d ** -0.5, rel,
                                                            talk, pb, gate, split_for=split, **tiles),
         kv_bytes, 4 * pairs * H * d, pairs * (2 * H * H + 8 * H))
-    if not decode:
-        put("sigmoid_attention, general kernel (what float32 runs)",
-            lambda: ops.sigmoid_attention(q, d, o, d, kp, vp, table, seq_of_token, positions, H, d ** -0.5, rel, talk, pb, gate),
-            kv_bytes, 0, pairs * (4 * H * d + 2 * H * H + 8 * H))
+    put("sigmoid_attention, general kernel (what float32 runs)",
+        lambda: ops.sigmoid_attention(q, d, o, d, kp, vp, table, seq_of_token, positions, H, d ** -0.5, rel, talk, pb, gate,
+                                      split_for=split if decode else 0), kv_bytes, 0, pairs * (4 * H * d + 2 * H * H + 8 * H))
     q_start = i32(list(range(0, rows + 1, rows // n_seqs)))
     put("paged_attention_general (the softmax attention's general kernel)",
         lambda: ops.paged_attention_general(q, o, kp, vp, table, seq_of_token, positions, H, d ** -0.5), kv_bytes, 4 * pairs * H * d)

@@ -71,7 +71,10 @@ __device__ __forceinline__ bf16x8 mask_slots(bf16x8 v, int ka, int hi) {
   return __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, v) & m);
 }
 
-template <int HPW>
+// KV1: the heads of a wave all belong to one kv head (the heads of a group are a multiple of a wave's heads).  Then
+// a wave keeps one set of key operands and one of value operands, and they are asked for ahead of their use: the
+// next tile's keys before the mixing of this one, this tile's values before its scores.
+template <int HPW, bool KV1>
 __global__ __launch_bounds__(ST_THREADS) void sigmoid_tile_kernel(const SigmoidTileArgs a) {
   extern __shared__ float lds[];
   float* raw = lds;                                          // [HP][KT][RAW_LD]
@@ -119,26 +122,72 @@ __global__ __launch_bounds__(ST_THREADS) void sigmoid_tile_kernel(const SigmoidT
 #pragma unroll
   for (int s = 0; s < HP / 4; ++s) talk_op[s] = a.talk[row * HP + 4 * s + g];
 
+  // A tile of 32 keys lies in one page (pages hold a multiple of 32 keys); keys of the tile beyond the item's last
+  // position may never have been written: whatever they hold, their weights are masked by a select.
+  const int my_kv = min(wave * HPW, H - 1) / rep;
+  bf16x8 kpre[KT / 16][NKS], vpre[NDB];
+  auto ask_keys = [&](int k0) {
+    const bf16_t* kp = a.k_pages + ((size_t)table[k0 / a.page_size] * a.n_kv + my_kv) * head_elems;
+#pragma unroll
+    for (int kb = 0; kb < KT / 16; ++kb)
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int dim = 32 * ks + 8 * g;
+        kpre[kb][ks] = dim < HD ? *(const bf16x8*)(kp + lay.k_off(k0 % a.page_size + 16 * kb + row, dim < HD ? dim : 0)) : zero8();
+      }
+  };
+  auto ask_values = [&](int k0) {
+    const bf16_t* vhead = a.v_pages + ((size_t)table[k0 / a.page_size] * a.n_kv + my_kv) * head_elems;
+    const int kc = (k0 % a.page_size) / 8 + g;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) vpre[db] = *(const bf16x8*)(vhead + lay.v_chunk_off(kc, 16 * db + row));
+  };
+  if (KV1) ask_keys(k_begin);
+
   for (int k0 = k_begin; k0 <= k_last; k0 += KT) {
     __syncthreads();  // raw is zeroed; the tile before is done with raw (and its weights are read below, after a barrier)
-    // ---- 1. scores
+    if (KV1) {
+      ask_values(k0);
+      // ---- 1. scores
 #pragma unroll
-    for (int j = 0; j < HPW; ++j) {
-      const int h = wave * HPW + j;
-      if (h < H) {  // uniform in the wave
-        const int kvh = h / rep;
+      for (int kb = 0; kb < KT / 16; ++kb)
 #pragma unroll
-        for (int kb = 0; kb < KT / 16; ++kb) {
-          const int key = min(k0 + 16 * kb + row, pos_last);  // a key that exists; those beyond a row's position are masked below
-          const bf16_t* kp = a.k_pages + ((size_t)table[key / a.page_size] * a.n_kv + kvh) * head_elems;
-          const int kappa = key % a.page_size;
+        for (int j = 0; j < HPW; ++j) {
+          const int h = wave * HPW + j;
+          if (h < H) {  // uniform in the wave
+            f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kpre[kb][ks], qop[j][ks], s, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) raw[(h * KT + 16 * kb + 4 * g + i) * RAW_LD + row] = s[i];
+          }
+        }
+      if (k0 + KT <= k_last) ask_keys(k0 + KT);
+    }
+    // ---- 1. scores (heads of one kv head that follow each other in a wave share its keys' operands)
+#pragma unroll
+    for (int kb = 0; kb < (KV1 ? 0 : KT / 16); ++kb) {
+      const int key = min(k0 + 16 * kb + row, pos_last);  // a key that exists; those beyond a row's position are masked below
+      const bf16_t* kpage = a.k_pages + (size_t)table[key / a.page_size] * a.n_kv * head_elems;
+      const int kappa = key % a.page_size;
+      bf16x8 kop[NKS];
+      int loaded = -1;
+#pragma unroll
+      for (int j = 0; j < HPW; ++j) {
+        const int h = wave * HPW + j;
+        if (h < H) {  // uniform in the wave
+          const int kvh = h / rep;
+          if (kvh != loaded) {  // uniform in the wave
+            loaded = kvh;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+              const int dim = 32 * ks + 8 * g;
+              kop[ks] = dim < HD ? *(const bf16x8*)(kpage + (size_t)kvh * head_elems + lay.k_off(kappa, dim < HD ? dim : 0)) : zero8();
+            }
+          }
           f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int ks = 0; ks < NKS; ++ks) {
-            const int dim = 32 * ks + 8 * g;
-            const bf16x8 k = dim < HD ? *(const bf16x8*)(kp + lay.k_off(kappa, dim < HD ? dim : 0)) : zero8();
-            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k, qop[j][ks], s, 0, 0, 0);
-          }
+          for (int ks = 0; ks < NKS; ++ks) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[ks], qop[j][ks], s, 0, 0, 0);
 #pragma unroll
           for (int i = 0; i < 4; ++i) raw[(h * KT + 16 * kb + 4 * g + i) * RAW_LD + row] = s[i];
         }
@@ -157,7 +206,7 @@ __global__ __launch_bounds__(ST_THREADS) void sigmoid_tile_kernel(const SigmoidT
       const f32x4 mb = *(const f32x4*)(a.mixed + (size_t)dist_c * HP + 4 * g);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float w = visible ? 1.f / (1.f + __expf(-(m[i] + mb[i]))) : 0.f;
+        const float w = visible ? __builtin_amdgcn_rcpf(1.f + __expf(-(m[i] + mb[i]))) : 0.f;  // (the reciprocal: one ulp)
         const __bf16 hi = (__bf16)w;
         const __bf16 lo = (__bf16)(w - (float)hi);
         wts[((4 * g + i) * TQ + row) * W_LD + kk] =
@@ -165,13 +214,28 @@ __global__ __launch_bounds__(ST_THREADS) void sigmoid_tile_kernel(const SigmoidT
       }
     }
     __syncthreads();
-    // ---- 3. values
+    // ---- 3. values (a kv head's operands are read once for the heads of its group that follow each other)
     const int page = table[k0 / a.page_size];
     const int kc = (k0 % a.page_size) / 8 + g;
+    bf16x8 vop[NDB];
+    int loaded = -1;
+    if (KV1) {
+      loaded = my_kv;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) vop[db] = mask_slots(vpre[db], k0 + 4 * g, pos_last);
+    }
 #pragma unroll
     for (int j = 0; j < HPW; ++j) {
       const int h = wave * HPW + j;
       if (h < H) {
+        const int kvh = h / rep;
+        if (kvh != loaded) {
+          loaded = kvh;
+          const bf16_t* vhead = a.v_pages + ((size_t)page * a.n_kv + kvh) * head_elems;
+#pragma unroll
+          for (int db = 0; db < NDB; ++db)  // a slot never written may hold anything: masked
+            vop[db] = mask_slots(*(const bf16x8*)(vhead + lay.v_chunk_off(kc, 16 * db + row)), k0 + 4 * g, pos_last);
+        }
         const uint32_t* wr = wts + (h * TQ + row) * W_LD;
         const u32x4 w0 = *(const u32x4*)(wr + 4 * g), w1 = *(const u32x4*)(wr + 16 + 4 * g);
         u32x4 hi, lo;  // eight bfloat16 each: keys 4g..4g+3 and 16+4g..16+4g+3
@@ -184,13 +248,10 @@ __global__ __launch_bounds__(ST_THREADS) void sigmoid_tile_kernel(const SigmoidT
         lo[2] = (w1[0] & 0xffffu) | (w1[1] << 16);
         lo[3] = (w1[2] & 0xffffu) | (w1[3] << 16);
         const bf16x8 p_hi = __builtin_bit_cast(bf16x8, hi), p_lo = __builtin_bit_cast(bf16x8, lo);
-        const bf16_t* vhead = a.v_pages + ((size_t)page * a.n_kv + h / rep) * head_elems;
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-          bf16x8 v = *(const bf16x8*)(vhead + lay.v_chunk_off(kc, 16 * db + row));
-          v = mask_slots(v, k0 + 4 * g, pos_last);  // a slot never written may hold anything
-          o[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p_hi, o[j][db], 0, 0, 0);
-          o[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p_lo, o[j][db], 0, 0, 0);
+          o[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[db], p_hi, o[j][db], 0, 0, 0);
+          o[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[db], p_lo, o[j][db], 0, 0, 0);
         }
       }
     }
@@ -251,16 +312,22 @@ extern "C" int fg_sigmoid_attention_tiles(const SigmoidTileArgs* args, hipStream
   const size_t lds = (size_t)HP * KT * RAW_LD * sizeof(float) + (size_t)HP * TQ * W_LD * sizeof(uint32_t);
   dim3 grid(a.n_items, a.n_chunks);
   const int hpw = (a.n_heads + 3) / 4;
-#define GO(HPW)                                                                                                       \
+#define GO1(HPW, KV1)                                                                                                 \
   do {                                                                                                                \
-    if (hipFuncSetAttribute((const void*)sigmoid_tile_kernel<HPW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) \
+    if (hipFuncSetAttribute((const void*)sigmoid_tile_kernel<HPW, KV1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) \
       return FG_ERR_LAUNCH;                                                                                           \
-    sigmoid_tile_kernel<HPW><<<grid, ST_THREADS, lds, stream>>>(a);                                                  \
+    sigmoid_tile_kernel<HPW, KV1><<<grid, ST_THREADS, lds, stream>>>(a);                                             \
+  } while (0)
+#define GO(HPW)                                       \
+  do {                                                \
+    if ((a.n_heads / a.n_kv) % HPW == 0) GO1(HPW, true); \
+    else GO1(HPW, false);                             \
   } while (0)
   if (hpw == 1) GO(1);
   else if (hpw == 2) GO(2);
   else GO(4);
 #undef GO
+#undef GO1
   if (a.partial)
     sigmoid_tile_combine_kernel<<<dim3(a.n_tokens, (a.n_heads * a.e + ST_THREADS - 1) / ST_THREADS), ST_THREADS, 0, stream>>>(a);
   return fg_launch_status();

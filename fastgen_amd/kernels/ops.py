@@ -1418,8 +1418,8 @@ class _SelectiveArgs(ctypes.Structure):
                 ("write_tail", ctypes.c_int), ("dsum", ctypes.c_void_p)]
 
 
-SELECTIVE_CHUNK = 64  # tokens of a chunk where long runs of tokens are scanned chunk by chunk, side by side
-SELECTIVE_CHUNKED_FROM = 192  # the shortest run of tokens of one sequence for which a step is scanned so
+SELECTIVE_CHUNK = 32  # tokens of a chunk where long runs of tokens are scanned chunk by chunk, side by side
+SELECTIVE_CHUNKED_FROM = 96  # the shortest run of tokens of one sequence for which a step is scanned so
 
 
 def _rows_of_width(t: torch.Tensor, T: int, width: int, name: str) -> None:
@@ -1572,7 +1572,7 @@ class _SigmoidTileArgs(ctypes.Structure):
 
 SIGMOID_TILE_TOKENS = 16  # query tokens of an item of the matrix-core kernel
 SIGMOID_TILE_HEADS = 16  # the most heads it mixes
-SIGMOID_TILE_CHUNK = 512  # keys of a chunk, at least; at most SIGMOID_TILE_MAX_CHUNKS chunks
+SIGMOID_TILE_CHUNK = 1024  # keys of a chunk, at least; at most SIGMOID_TILE_MAX_CHUNKS chunks
 SIGMOID_TILE_MAX_CHUNKS = 8
 SIGMOID_TILE_FEW_TOKENS = 64  # up to so many tokens a step, chunks of SIGMOID_TILE_FEW_CHUNK keys, as many as it takes
 SIGMOID_TILE_FEW_CHUNK = 128
