@@ -164,7 +164,9 @@ def _paged(T, n_kv, hc, P, dtype, seed):
 @pytest.mark.parametrize("H,G,d,e,hc,P,rows,far,every,T", [(4, 2, 6, 4, 8, 8, 6, 9.0, 3, 29), (8, 4, 80, 48, 80, 64, 24, 150.0, 100, 700),
                                                             (3, 3, 8, 10, 16, 16, 8, 40.0, 1, 150), (34, 2, 8, 8, 16, 16, 64, 33.0, 7, 90),
                                                             (5, 1, 20, 48, 48, 32, 9, 1000.0, 1000, 300),
-                                                            (16, 4, 64, 64, 64, 64, 16, 600.0, 50, 1100), (12, 3, 32, 16, 32, 32, 10, 64.0, 9, 130)])
+                                                            (16, 4, 64, 64, 64, 64, 16, 600.0, 50, 1100), (12, 3, 32, 16, 32, 32, 10, 64.0, 9, 130),
+                                                            (12, 4, 16, 16, 16, 32, 12, 90.0, 4, 200), (16, 16, 32, 32, 32, 64, 8, 20.0, 11, 150),
+                                                            (3, 3, 8, 10, 16, 32, 8, 40.0, 1, 100), (1, 1, 24, 8, 32, 96, 6, 7.0, 2, 250)])
 def test_prepare_and_sigmoid_attention_kernels(dtype, H, G, d, e, hc, P, rows, far, every, T):
     """Unit norms per head, the query's temperature, blended values, pages; then the attention over the pages for
     a whole prompt, for its last tokens alone with the keys cut over workgroups, and both with the same bits."""
