@@ -195,7 +195,9 @@ __global__ __launch_bounds__(ST_THREADS) void sigmoid_tile_kernel(const SigmoidT
     }
     __syncthreads();
     // ---- 2. mixing, bias, sigmoid, mask: a wave a key in turns; a lane ends with 4 heads of a (token, key)
-    for (int kk = wave; kk < KT; kk += ST_THREADS / FG_WAVE) {
+#pragma unroll  // (eight keys a wave: their chains of reads, products and exponentials run side by side)
+    for (int kq = 0; kq < KT / (ST_THREADS / FG_WAVE); ++kq) {
+      const int kk = wave + kq * (ST_THREADS / FG_WAVE);
       f32x4 m = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < HP / 4; ++s)

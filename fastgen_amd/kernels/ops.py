@@ -1574,7 +1574,7 @@ SIGMOID_TILE_TOKENS = 16  # query tokens of an item of the matrix-core kernel
 SIGMOID_TILE_HEADS = 16  # the most heads it mixes
 SIGMOID_TILE_CHUNK = 1024  # keys of a chunk, at least; at most SIGMOID_TILE_MAX_CHUNKS chunks
 SIGMOID_TILE_MAX_CHUNKS = 8
-SIGMOID_TILE_FEW_TOKENS = 64  # up to so many tokens a step, chunks of SIGMOID_TILE_FEW_CHUNK keys, as many as it takes
+SIGMOID_TILE_FEW_TOKENS = 64  # up to so many tokens a step, chunks of SIGMOID_TILE_FEW_CHUNK keys or more, as many as it takes
 SIGMOID_TILE_FEW_CHUNK = 128
 
 
@@ -1636,8 +1636,8 @@ def _sigmoid_attention_tiles(q, head_dim, out, v_head_dim, k_pages, v_pages, blo
               and gate.shape[1] >= H, "gate must be float32 [T, >= H]")
         a.gate, a.gate_stride = gate.data_ptr(), gate.stride(0)
     max_keys = max(int(max_keys), 1)
-    if T <= SIGMOID_TILE_FEW_TOKENS:  # decoding: many small chunks, so that few tokens fill the device
-        chunk = SIGMOID_TILE_FEW_CHUNK
+    if T <= SIGMOID_TILE_FEW_TOKENS:  # decoding: small chunks, so that few tokens give a workgroup for every compute unit
+        chunk = min(SIGMOID_TILE_CHUNK, max(SIGMOID_TILE_FEW_CHUNK, -(-T * max_keys // (compute_units() * 32)) * 32))
     else:
         chunk = max(SIGMOID_TILE_CHUNK, -(-max_keys // (SIGMOID_TILE_MAX_CHUNKS * 32)) * 32)
     n_chunks = -(-max_keys // chunk)
