@@ -91,6 +91,13 @@ template <class TA> __device__ __forceinline__ float fast_exp(float x);
 template <> __device__ __forceinline__ float fast_exp<float>(float x) { return expf(x); }
 // bfloat16 operands: the hardware's exponential (a few ulp of 32-bit)
 template <> __device__ __forceinline__ float fast_exp<bf16_t>(float x) { return __expf(x); }
+// softplus and the sigmoid of the gate: exact functions for 32-bit operands, the hardware's for bfloat16
+template <class TA> __device__ __forceinline__ float softplus_of(float d);
+template <> __device__ __forceinline__ float softplus_of<float>(float d) { return d > 20.f ? d : log1pf(expf(d)); }
+template <> __device__ __forceinline__ float softplus_of<bf16_t>(float d) { return d > 20.f ? d : __logf(1.f + __expf(d)); }
+template <class TA> __device__ __forceinline__ float silu_of(float z);
+template <> __device__ __forceinline__ float silu_of<float>(float z) { return z / (1.f + expf(-z)); }
+template <> __device__ __forceinline__ float silu_of<bf16_t>(float z) { return z * __builtin_amdgcn_rcpf(1.f + __expf(-z)); }
 
 template <class TA, class TD, int SPL, bool OUT>
 __global__ __launch_bounds__(SS_THREADS) void selective_scan_kernel(const ScanArgs a) {
@@ -140,7 +147,7 @@ __global__ __launch_bounds__(SS_THREADS) void selective_scan_kernel(const ScanAr
 #pragma unroll
     for (int i = 0; i < SPL; ++i) { Bv[i] = n_B[i]; Cv[i] = n_C[i]; }
     if (t + 1 < t1) fetch(t + 1);
-    d = d > 20.f ? d : log1pf(expf(d));  // softplus
+    d = softplus_of<TA>(d);
     d_total += d;
     const float du = d * uv;
     float y = 0.f;
@@ -153,7 +160,7 @@ __global__ __launch_bounds__(SS_THREADS) void selective_scan_kernel(const ScanAr
       for (int m = 1; m < a.LP; m <<= 1) y += __shfl_xor(y, m, FG_WAVE);
       if (g == 0 && live) {
         y = fmaf(skip, uv, y);
-        if (z) y *= zv / (1.f + fast_exp<TA>(-zv));
+        if (z) y *= silu_of<TA>(zv);
         out[(size_t)t * a.ldo] = from_f<TA>(y);
       }
     }
