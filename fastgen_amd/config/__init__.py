@@ -11,6 +11,7 @@ from . import llama as _llama  # registers LlamaForCausalLM
 from . import buderax as _buderax  # registers Buderax
 from . import gisodra as _gisodra  # registers Gisodra
 from . import zudisun as _zudisun  # registers Zudisun
+from . import sodotar as _sodotar  # registers Sodotar
 
 __all__ = [
     "Architecture",

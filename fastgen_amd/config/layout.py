@@ -34,7 +34,9 @@ class LayerSpec:
     one whose sublayers share the mixer's norm (the arrangement must know).
     ``extra_norms``: further norms by name, for arrangements that own more
     than two (norms after the mixer and the feed-forward, say); the
-    arrangement gets them as a dict."""
+    arrangement gets them as a dict.  ``arrangement_spec``: for an arrangement
+    with sizes, constants or tensors of its own (its kind is then the
+    arrangement's name); it is a part like the others."""
 
     mixer: PartSpec
     ffn: Optional[PartSpec]
@@ -42,6 +44,7 @@ class LayerSpec:
     ffn_norm: Optional[PartSpec]
     arrangement: str = "pre_norm"
     extra_norms: Mapping[str, PartSpec] = field(default_factory=dict)
+    arrangement_spec: Optional[PartSpec] = None
 
 
 @dataclass(frozen=True)
@@ -73,8 +76,13 @@ class ModelLayout:
     final_norm: PartSpec
     head: PartSpec
     injections: Tuple[PartSpec, ...] = ()
+    # S >= 1: the model keeps S residual streams side by side, fp32 [S, T, dim]: the embedding's output is copied
+    # into each, the layers' arrangements update them, the last norm reads their sum; 0: the one plain stream [T, dim]
+    streams: int = 0
 
     def __post_init__(self) -> None:
+        if self.streams and self.injections:
+            raise ValueError("injections add to the one plain residual stream: a model of several streams has none")
         for i, e in enumerate(self.order):
             if e.inject is not None and not 0 <= e.inject[0] < len(self.injections):
                 raise ValueError(f"order[{i}] names injection {e.inject[0]}, which does not exist")

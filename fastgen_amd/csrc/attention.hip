@@ -58,7 +58,7 @@ __global__ __launch_bounds__(ATT_WAVES* FG_WAVE) void paged_attention_general_ke
   const int seq = seq_of_token[t];
   const int pos = positions[t];
   const int* table = block_table + (size_t)seq * bt_stride;
-  const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+  const int first = first_key(pos, window);
   const KvLayout lay(page_size, hd);
   const size_t head_elems = (size_t)page_size * hd;
 
@@ -150,7 +150,7 @@ extern "C" int fg_paged_attention_general_sink(
     float scale, int window, const float* sinks, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
   if (hd <= 0 || hd % 8 || hd > ATT_MAX_HD || page_size <= 0 || page_size % 8 || n_kv <= 0 ||
-      n_heads <= 0 || n_heads % n_kv || window < 0)
+      n_heads <= 0 || n_heads % n_kv)
     return FG_ERR_ARG;
   const long long items = (long long)n_tokens * n_heads;
   const long long blocks = (items + ATT_WAVES - 1) / ATT_WAVES;

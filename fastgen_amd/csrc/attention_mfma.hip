@@ -245,7 +245,7 @@ constexpr int PLAN_HEAD = 4;
 // tiles an item's rows see: [t_lo, t_hi]
 __device__ __forceinline__ void item_tiles(const Item& it, int window, int& t_lo, int& t_hi) {
   const int pos_last = it.pos0 + it.n_tok - 1;
-  const int first_min = window > 0 && it.pos0 - window + 1 > 0 ? it.pos0 - window + 1 : 0;
+  const int first_min = first_key(it.pos0, window);
   t_lo = first_min / TILE;
   t_hi = pos_last / TILE;
 }
@@ -371,13 +371,13 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
   const KvLayout lay(page_size, HD);
 
   const int pos_last = it.pos0 + it.n_tok - 1;
-  const int first_min = window > 0 && it.pos0 - window + 1 > 0 ? it.pos0 - window + 1 : 0;
+  const int first_min = first_key(it.pos0, window);
   ItemRows me[1] = {{-1, 0}};
   const bool my_row = r16 < it.n_tok * G;
   const int my_tok = my_row ? r16 / G : 0, my_head = my_row ? r16 % G : 0;
   if (my_row) {
     me[0].pos = it.pos0 + my_tok;
-    me[0].first = window > 0 && me[0].pos - window + 1 > 0 ? me[0].pos - window + 1 : 0;
+    me[0].first = first_key(me[0].pos, window);
   }
   bf16x8 qop[1][NKS];
   load_q(qop[0], q + (size_t)(it.tok0 + my_tok) * q_stride + (size_t)(kvh * G + my_head) * HD, my_row);
@@ -666,7 +666,7 @@ extern "C" long long fg_attn_plan_ints(int max_chunks) { return PLAN_HEAD + 8LL 
 extern "C" int fg_attn_plan(const int* items, int n_items, int window, int max_chunks, int min_tiles, int* plan,
                             hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
-  if (!items || !plan || max_chunks < 2 * n_items || min_tiles < 1 || window < 0) return FG_ERR_ARG;
+  if (!items || !plan || max_chunks < 2 * n_items || min_tiles < 1) return FG_ERR_ARG;
   attn_plan_kernel<<<1, 256, 0, stream>>>(items, n_items, window, max_chunks, min_tiles, plan);
   return fg_launch_status();
 }
@@ -683,7 +683,7 @@ extern "C" int fg_attn_split_sink(const void* q, int q_stride, void* out, int ou
                                   const float* sinks, hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
   if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || page_size < 8 || page_size % 8 ||
-      !(scale > 0.f) || max_chunks < 2 * n_items || max_chunks > 65535 || n_kv > 65535 || window < 0 ||
+      !(scale > 0.f) || max_chunks < 2 * n_items || max_chunks > 65535 || n_kv > 65535 ||
       q_stride % 8 || out_stride % 4 || !plan || !part_o || !part_ml || max_rows < 1 || max_rows > 16)
     return FG_ERR_ARG;
 #define LAUNCH(PERM)                                                                                           \
@@ -837,7 +837,7 @@ __global__ __launch_bounds__(TILE_PAIR ? 512 : 256, TILE_PAIR ? 1 : 2) void attn
   const Pager pager{block_table + (size_t)it.seq * bt_stride, page_size, page_shift};
   const KvLayout lay(page_size, HD);
   const int pos_last = it.pos0 + it.n_tok - 1;
-  const int first_min = window > 0 && it.pos0 - window + 1 > 0 ? it.pos0 - window + 1 : 0;
+  const int first_min = first_key(it.pos0, window);
 
   constexpr int RB = TILE_RB;
   ItemRows me[RB];
@@ -852,7 +852,7 @@ __global__ __launch_bounds__(TILE_PAIR ? 512 : 256, TILE_PAIR ? 1 : 2) void attn
     me[rb] = ItemRows{-1, 0};
     if (my_row) {
       me[rb].pos = it.pos0 + my_tok;
-      me[rb].first = window > 0 && me[rb].pos - window + 1 > 0 ? me[rb].pos - window + 1 : 0;
+      me[rb].first = first_key(me[rb].pos, window);
       w_hi = max(w_hi, me[rb].pos);
       w_lo = min(w_lo, me[rb].first);
       w_all_hi = min(w_all_hi, me[rb].pos);
@@ -1115,7 +1115,7 @@ extern "C" int fg_attn_tile_sink(const void* q, int q_stride, void* out, int out
                                  float scale, int window, const float* sinks, hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
   if (hd != HD || !(scale > 0.f) || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > item_rows || page_size < 8 || page_size % 8 ||
-      (long long)n_items * n_kv > 2147483647LL || window < 0 || q_stride % 8 || out_stride % 4 ||
+      (long long)n_items * n_kv > 2147483647LL || q_stride % 8 || out_stride % 4 ||
       (item_rows != TILE_ROWS && item_rows != TILE_ROWS_SMALL))
     return FG_ERR_ARG;
   const TileArgs a{(const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,

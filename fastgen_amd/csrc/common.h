@@ -97,6 +97,36 @@ __device__ __forceinline__ float block_max(float v, float* lds) {
   return total;
 }
 
+// The first key that a query at position `pos` sees (the last one is `pos` itself).  span > 0: a sliding
+// window of `span` keys; span < 0: the keys of the query's own block of -span positions, blocks counted from
+// position 0 of the sequence; 0: every key from 0 on.  Never decreases as pos grows.
+__host__ __device__ __forceinline__ int first_key(int pos, int span) {
+  if (span > 0) return pos - span + 1 > 0 ? pos - span + 1 : 0;
+  if (span < 0) return pos - pos % (-span);
+  return 0;
+}
+
+// The gated activations of the routed and dense feed-forwards: kind 0 is silu(g) * u; kind 3 limits both
+// halves first, g = min(g, limit), u = clamp(u, -limit, limit), and gives g * sigmoid(alpha * g) * (u + 1).
+// (Kinds 1 and 2, the tanh form of GELU and ReLU, exist in the dense kernels only.)
+#define FG_ACT_SILU 0
+#define FG_ACT_LIMITED 3
+struct GatedAct {
+  int kind;
+  float limit, alpha;
+};
+template <bool FAST>
+__device__ __forceinline__ float gated_act(float g, float u, const GatedAct a) {
+  if (a.kind == FG_ACT_LIMITED) {
+    g = fminf(g, a.limit);
+    u = fminf(fmaxf(u, -a.limit), a.limit);
+    const float e = FAST ? __expf(-a.alpha * g) : expf(-a.alpha * g);
+    return (FAST ? g * __frcp_rn(1.f + e) : g / (1.f + e)) * (u + 1.f);
+  }
+  const float e = FAST ? __expf(-g) : expf(-g);
+  return (FAST ? g * __frcp_rn(1.f + e) : g / (1.f + e)) * u;
+}
+
 static inline int fg_launch_status() {
   return hipGetLastError() == hipSuccess ? FG_OK : FG_ERR_LAUNCH;
 }

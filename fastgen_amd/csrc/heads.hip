@@ -9,6 +9,7 @@
 //  head_linear     y[t, h, :] = W_h x[t, h, :] with a matrix per head, an optional sigmoid gate per
 //                  (token, head), and a run of x's columns behind the product's copied through.
 //  head_norm_gate  RMS norm per head of fp32 rows times silu(gate).
+//  head_diff_norm  the difference of two attention maps' outputs per head, divided by its root mean square.
 //
 // All arithmetic between a load and a store is fp32; a result is rounded once, at the store.
 #include "common.h"
@@ -337,6 +338,59 @@ extern "C" int fg_head_norm_gate(const float* x, const float* w, const void* gat
   else if (act_dtype == FG_BF16)
     head_norm_gate_kernel<bf16_t><<<grid, HP_WAVES * FG_WAVE, 0, stream>>>(x, w, (const bf16_t*)gate, gate_stride,
                                                                           (bf16_t*)out, H, e, eps);
+  else
+    return FG_ERR_ARG;
+  return fg_launch_status();
+}
+
+// ---------------------------------------------------------------- head_diff_norm
+// Two attention maps a head, one value: out[t, h, :] = n(a1 - lam * a2) * out_scale with
+// n(o) = o * rsqrt(mean(o^2) + eps) over the head's e values (no weight).  `att` holds 2 H heads of `hw`
+// columns (the first e are the head's output): the heads of a key/value group of `group` query heads lie
+// as [map 1 of the group's heads | map 2 of the group's heads], so a1 of head h is head
+// (h / group) * 2 * group + h % group of `att` and a2 lies `group` heads behind it.  All in fp32, one
+// rounding at the store.  grid (T, ceil(H / 4)); a wave a (token, head).
+template <class TA>
+__global__ __launch_bounds__(HP_WAVES* FG_WAVE) void head_diff_norm_kernel(
+    const TA* __restrict__ att, int att_stride, int hw, TA* __restrict__ out, int out_stride, int H, int group, int e,
+    float lam, float eps, float out_scale) {
+  const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
+  const int t = blockIdx.x, h = blockIdx.y * HP_WAVES + wave;
+  if (h >= H) return;
+  const TA* a1 = att + (size_t)t * att_stride + (size_t)((h / group) * 2 * group + h % group) * hw;
+  const TA* a2 = a1 + (size_t)group * hw;
+  float v[HN_MAX];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < HN_MAX; ++j) {
+    const int d = lane + FG_WAVE * j;
+    v[j] = d < e ? to_f<TA>(a1[d]) - lam * to_f<TA>(a2[d]) : 0.f;
+    ss += v[j] * v[j];
+  }
+  ss = wave_sum(ss);
+  const float mul = rsqrtf(ss / (float)e + eps) * out_scale;
+  TA* o = out + (size_t)t * out_stride + (size_t)h * e;
+#pragma unroll
+  for (int j = 0; j < HN_MAX; ++j) {
+    const int d = lane + FG_WAVE * j;
+    if (d < e) o[d] = from_f<TA>(v[j] * mul);
+  }
+}
+
+extern "C" int fg_head_diff_norm(const void* att, int att_stride, int hw, void* out, int out_stride, int n_tokens, int H,
+                                 int group, int e, float lam, float eps, float out_scale, int act_dtype,
+                                 hipStream_t stream) {
+  if (n_tokens <= 0) return FG_OK;
+  if (H <= 0 || group <= 0 || H % group || e <= 0 || e > HN_MAX * FG_WAVE || hw < e || att_stride < 2 * H * hw ||
+      out_stride < H * e || (H + HP_WAVES - 1) / HP_WAVES > 65535)
+    return FG_ERR_ARG;
+  dim3 grid(n_tokens, (H + HP_WAVES - 1) / HP_WAVES);
+  if (act_dtype == FG_F32)
+    head_diff_norm_kernel<float><<<grid, HP_WAVES * FG_WAVE, 0, stream>>>((const float*)att, att_stride, hw, (float*)out,
+                                                                         out_stride, H, group, e, lam, eps, out_scale);
+  else if (act_dtype == FG_BF16)
+    head_diff_norm_kernel<bf16_t><<<grid, HP_WAVES * FG_WAVE, 0, stream>>>((const bf16_t*)att, att_stride, hw, (bf16_t*)out,
+                                                                          out_stride, H, group, e, lam, eps, out_scale);
   else
     return FG_ERR_ARG;
   return fg_launch_status();

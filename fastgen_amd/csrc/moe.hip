@@ -31,12 +31,18 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // score plus `correction` (per expert, or null), inside the `keep_groups` best of `n_groups` groups of
 // neighbouring experts (a group's rank: the sum of its two largest choice scores; the experts of the other
 // groups cannot be chosen); the weights are the chosen experts' scores without the correction, divided by
-// their sum (+ 1e-20) and multiplied by `weight_scale`.
+// their sum (+ 1e-20) and multiplied by `weight_scale`.  A third way (`sigmoid_scores` = 2): the scores are the
+// softmax of the logits over all experts; choice, groups and weights as with sigmoid scores.
+//
+// `n_extra`: the router matrix has that many rows more than there are experts; their logits (no bias) take no
+// part in the choice and are stored as they are in `extra [n_tokens, n_extra]` (a gate of a shared expert, say).
 struct RouteMode {
   int sigmoid_scores;
   const float* correction;
   int n_groups, keep_groups;
   float weight_scale;
+  int n_extra;
+  float* extra;
 };
 template <class T, int WAVES, int EPW>
 __global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
@@ -44,12 +50,13 @@ __global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
     int dim, int n_experts, int top, int* __restrict__ choice, float* __restrict__ weight, const RouteMode mode) {
   extern __shared__ float lds[];
   float* z = lds;
-  float* chosen = lds + n_experts;
+  float* chosen = lds + n_experts + mode.n_extra;
+  const int n_rows = n_experts + mode.n_extra;  // rows of the router matrix
   float* score = chosen + top;
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const size_t t = blockIdx.x;
   const T* xr = x + t * ldx;
-  for (int e0 = wave * EPW; e0 < n_experts; e0 += WAVES * EPW) {
+  for (int e0 = wave * EPW; e0 < n_rows; e0 += WAVES * EPW) {
     float s[EPW];
 #pragma unroll
     for (int j = 0; j < EPW; ++j) s[j] = 0.f;
@@ -60,7 +67,7 @@ __global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
 #pragma unroll
         for (int j = 0; j < EPW; ++j) {
           float wv[8];
-          load8<float>(wr + (size_t)min(e0 + j, n_experts - 1) * dim + k, wv);
+          load8<float>(wr + (size_t)min(e0 + j, n_rows - 1) * dim + k, wv);
 #pragma unroll
           for (int i = 0; i < 8; ++i) s[j] = fmaf(xv[i], wv[i], s[j]);
         }
@@ -69,19 +76,29 @@ __global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
       for (int k = lane; k < dim; k += FG_WAVE) {
         const float xv = to_f<T>(xr[k]);
 #pragma unroll
-        for (int j = 0; j < EPW; ++j) s[j] = fmaf(xv, wr[(size_t)min(e0 + j, n_experts - 1) * dim + k], s[j]);
+        for (int j = 0; j < EPW; ++j) s[j] = fmaf(xv, wr[(size_t)min(e0 + j, n_rows - 1) * dim + k], s[j]);
       }
     }
 #pragma unroll
     for (int j = 0; j < EPW; ++j) {
       const float v = wave_sum(s[j]);
-      if (lane == 0 && e0 + j < n_experts) z[e0 + j] = v + (bias ? bias[e0 + j] : 0.f);
+      if (lane == 0 && e0 + j < n_rows) z[e0 + j] = v + (bias && e0 + j < n_experts ? bias[e0 + j] : 0.f);
     }
   }
   __syncthreads();
+  for (int e = threadIdx.x; e < mode.n_extra; e += blockDim.x) mode.extra[t * mode.n_extra + e] = z[n_experts + e];
   if (mode.sigmoid_scores) {  // uniform
+    float top_z = 0.f, all = 1.f;
+    if (mode.sigmoid_scores == 2) {
+      // every thread takes the maximum and the sum over all experts itself, in the experts' order
+      top_z = -INFINITY;
+      for (int e = 0; e < n_experts; ++e) top_z = fmaxf(top_z, z[e]);
+      all = 0.f;
+      for (int e = 0; e < n_experts; ++e) all += expf(z[e] - top_z);
+      __syncthreads();  // every thread has read the logits before any of them is overwritten
+    }
     for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
-      const float sc = 1.f / (1.f + expf(-z[e]));
+      const float sc = mode.sigmoid_scores == 2 ? expf(z[e] - top_z) / all : 1.f / (1.f + expf(-z[e]));
       score[e] = sc;
       z[e] = sc + (mode.correction ? mode.correction[e] : 0.f);
     }
@@ -151,14 +168,15 @@ __global__ __launch_bounds__(64 * WAVES) void moe_route_kernel(
 extern "C" int fg_moe_route_mode(const void* x, int ldx, int dtype, const float* wr, const float* bias, int n_tokens,
                                  int dim, int n_experts, int top, int* choice, float* weight, int sigmoid_scores,
                                  const float* correction, int n_groups, int keep_groups, float weight_scale,
-                                 hipStream_t stream) {
+                                 int n_extra, float* extra, hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
+  if (sigmoid_scores < 0 || sigmoid_scores > 2 || n_extra < 0 || (n_extra > 0 && !extra)) return FG_ERR_ARG;
   if (dim <= 0 || ldx < dim || n_experts <= 0 || top < 1 || top > n_experts) return FG_ERR_ARG;
   if (n_groups < 1 || n_experts % n_groups || keep_groups < 1 || keep_groups > n_groups ||
       top > keep_groups * (n_experts / n_groups) || (!sigmoid_scores && (correction || n_groups > 1)))
     return FG_ERR_ARG;
-  const RouteMode mode = {sigmoid_scores, correction, n_groups, keep_groups, weight_scale};
-  const size_t lds = (size_t)(2 * n_experts + top + n_groups) * sizeof(float);
+  const RouteMode mode = {sigmoid_scores, correction, n_groups, keep_groups, weight_scale, n_extra, extra};
+  const size_t lds = (size_t)(2 * n_experts + n_extra + top + n_groups) * sizeof(float);
   if (lds > 60000) return FG_ERR_ARG;
 #define GO(T, WAVES, EPW)                                                                                        \
   moe_route_kernel<T, WAVES, EPW><<<n_tokens, 64 * WAVES, lds, stream>>>((const T*)x, ldx, wr, bias, dim, n_experts, \
@@ -178,7 +196,7 @@ extern "C" int fg_moe_route_mode(const void* x, int ldx, int dtype, const float*
 extern "C" int fg_moe_route(const void* x, int ldx, int dtype, const float* wr, const float* bias, int n_tokens, int dim,
                             int n_experts, int top, int* choice, float* weight, hipStream_t stream) {
   return fg_moe_route_mode(x, ldx, dtype, wr, bias, n_tokens, dim, n_experts, top, choice, weight, 0, nullptr, 1, 1, 1.f,
-                           stream);
+                           0, nullptr, stream);
 }
 
 // -------------------------------------------------------------------- sort
@@ -264,7 +282,7 @@ template <class T>
 __global__ __launch_bounds__(256) void moe_gate_up_generic_kernel(
     const T* __restrict__ x, int ldx, const T* __restrict__ wg, const T* __restrict__ wu, int ldw /* row stride of wg, wu */,
     const int* __restrict__ sorted, const int* __restrict__ tiles, int top, int dim, int hidden, T* __restrict__ act,
-    int lda) {
+    int lda, const GatedAct fn) {
   const int4 tile = *(const int4*)(tiles + 4 * (size_t)blockIdx.x);
   const int r = threadIdx.x / 16, c = blockIdx.y * 16 + threadIdx.x % 16;
   if (r >= tile.z || c >= hidden) return;
@@ -272,7 +290,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_generic_kernel(
   const T* xr = x + (size_t)(sorted[pos] / top) * ldx;
   const size_t wrow = ((size_t)tile.x * hidden + c) * ldw;
   const float g = dot_ordered<T>(xr, wg + wrow, dim), u = dot_ordered<T>(xr, wu + wrow, dim);
-  act[(size_t)pos * lda + c] = from_f<T>(g / (1.f + expf(-g)) * u);
+  act[(size_t)pos * lda + c] = from_f<T>(gated_act<false>(g, u, fn));
 }
 
 template <class T>
@@ -305,7 +323,7 @@ template <int MB>
 __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ wg, const bf16_t* __restrict__ wu, int ldw,
     const int* __restrict__ sorted, const int* __restrict__ tiles, int max_tiles, int top, int dim, int hidden,
-    bf16_t* __restrict__ act, int lda) {
+    bf16_t* __restrict__ act, int lda, const GatedAct fn) {
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int cblocks = (hidden + 15) / 16;
   const int item = blockIdx.x * 4 + wave;
@@ -356,8 +374,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(
     bf16x4 o;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float gv = ag[mb][i];
-      o[i] = (__bf16)(gv * __frcp_rn(1.f + __expf(-gv)) * au[mb][i]);
+      o[i] = (__bf16)gated_act<true>(ag[mb][i], au[mb][i], fn);
     }
     bf16_t* dst = act + (size_t)(tile.y + r) * lda + c;
     if (c + 3 < hidden) {
@@ -435,7 +452,7 @@ template <int WM, int NST, int EPI>
 __global__ __launch_bounds__(128 * WM) void moe_tiled_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w0, const bf16_t* __restrict__ w1, int ldw,
     void* __restrict__ y, int ldy, const int* __restrict__ sorted, const int* __restrict__ tiles, int top,
-    int N /* rows of the matrix as the tile sees it: 2 * hidden (gate_up), dim (down) */, int K) {
+    int N /* rows of the matrix as the tile sees it: 2 * hidden (gate_up), dim (down) */, int K, const GatedAct fn) {
   constexpr int WN = 2, NW = WM * WN, WB = 4 * WN, XB = 4 * WM, NB = WB + XB, LPW = NB / NW, BLOCK = 16 * 32;
   static_assert(NB % NW == 0 && NST >= 3 && LPW * (NST - 2) < 64, "blocks divide over the waves; loads fit the counter");
   extern __shared__ __attribute__((aligned(16))) bf16_t ring[];  // [NST][NB][BLOCK]
@@ -529,7 +546,7 @@ __global__ __launch_bounds__(128 * WM) void moe_tiled_kernel(
         for (int i = 0; i < 4; ++i) {
           const float up = __shfl_xor(acc[mb][nb][i], 32, FG_WAVE);
           const float gate = acc[mb][nb][i];
-          v[i] = (__bf16)(gate * __frcp_rn(1.f + __expf(-gate)) * up);
+          v[i] = (__bf16)gated_act<true>(gate, up, fn);
         }
         if (g < 2 && valid && n0 + 15 < N) *(bf16x4*)((bf16_t*)y + (size_t)pos * ldy + n0 / 2 + 4 * g) = v;
       }
@@ -539,7 +556,8 @@ __global__ __launch_bounds__(128 * WM) void moe_tiled_kernel(
 
 template <int WM, int EPI>
 static int launch_moe_tiled(const void* x, int ldx, const void* w0, const void* w1, int ldw, void* y, int ldy,
-                            const int* sorted, const int* tiles, int max_tiles, int top, int N, int K, hipStream_t stream) {
+                            const int* sorted, const int* tiles, int max_tiles, int top, int N, int K, const GatedAct fn,
+                            hipStream_t stream) {
   constexpr int NST = 4, lds = NST * 4 * (WM + 2) * 1024;
   static bool raised = false;  // more than 64 KB of dynamic LDS has to be asked for once
   auto kernel = moe_tiled_kernel<WM, NST, EPI>;
@@ -551,31 +569,35 @@ static int launch_moe_tiled(const void* x, int ldx, const void* w0, const void* 
   if (max_tiles > 65535) return FG_ERR_ARG;
   const dim3 grid((N + 127) / 128, max_tiles);
   kernel<<<grid, 128 * WM, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w0, (const bf16_t*)w1, ldw, y, ldy, sorted,
-                                          tiles, top, N, K);
+                                          tiles, top, N, K, fn);
   return fg_launch_status();
 }
 
 // x [T, dim] rows gathered by token; wg, wu [E, hidden, ldw], act [n_pairs, lda] in the sorted order.
 // mfma: bf16 with dim % 8 == 0, ldx % 8 == 0, ldw % 8 == 0 (16-byte loads); tile_rows = 16 * MB, MB in 1, 2, 4,
 // or 128 / 256: the tiles that go through LDS.
-extern "C" int fg_moe_gate_up(const void* x, int ldx, const void* wg, const void* wu, int ldw, const int* sorted,
-                              const int* tiles, int max_tiles, int tile_rows, int top, int dim, int hidden, void* act,
-                              int lda, int dtype, int mfma, hipStream_t stream) {
+// act_kind, limit, alpha: the gated activation (GatedAct in common.h).
+extern "C" int fg_moe_gate_up_act(const void* x, int ldx, const void* wg, const void* wu, int ldw, const int* sorted,
+                                  const int* tiles, int max_tiles, int tile_rows, int top, int dim, int hidden, void* act,
+                                  int lda, int dtype, int mfma, int act_kind, float limit, float alpha,
+                                  hipStream_t stream) {
   if (max_tiles <= 0) return FG_OK;
+  if (act_kind != FG_ACT_SILU && !(act_kind == FG_ACT_LIMITED && limit > 0.f)) return FG_ERR_ARG;
+  const GatedAct fn = {act_kind, limit, alpha};
   if (dim <= 0 || hidden <= 0 || top <= 0 || ldx < dim || ldw < dim || lda < hidden) return FG_ERR_ARG;
   if (mfma) {
     if (dtype != FG_BF16 || dim % 8 || ldx % 8 || ldw % 8 || lda % 4) return FG_ERR_ARG;
     if (tile_rows == 128 || tile_rows == 256) {
       if (hidden % 8 || dim < 32) return FG_ERR_ARG;  // (a lane's stand-in load reads the row's first 32 k)
       return tile_rows == 128
-                 ? launch_moe_tiled<2, MT_GATE_UP>(x, ldx, wg, wu, ldw, act, lda, sorted, tiles, max_tiles, top, 2 * hidden, dim, stream)
-                 : launch_moe_tiled<4, MT_GATE_UP>(x, ldx, wg, wu, ldw, act, lda, sorted, tiles, max_tiles, top, 2 * hidden, dim, stream);
+                 ? launch_moe_tiled<2, MT_GATE_UP>(x, ldx, wg, wu, ldw, act, lda, sorted, tiles, max_tiles, top, 2 * hidden, dim, fn, stream)
+                 : launch_moe_tiled<4, MT_GATE_UP>(x, ldx, wg, wu, ldw, act, lda, sorted, tiles, max_tiles, top, 2 * hidden, dim, fn, stream);
     }
     const long long items = (long long)max_tiles * ((hidden + 15) / 16);
     const unsigned blocks = (unsigned)((items + 3) / 4);
 #define GO(MB)                                                                                                   \
   moe_gate_up_mfma_kernel<MB><<<blocks, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)wg, (const bf16_t*)wu, \
-                                                          ldw, sorted, tiles, max_tiles, top, dim, hidden, (bf16_t*)act, lda)
+                                                          ldw, sorted, tiles, max_tiles, top, dim, hidden, (bf16_t*)act, lda, fn)
     if (tile_rows == 16) GO(1);
     else if (tile_rows == 32) GO(2);
     else if (tile_rows == 64) GO(4);
@@ -588,14 +610,21 @@ extern "C" int fg_moe_gate_up(const void* x, int ldx, const void* wg, const void
   if (grid.y > 65535) return FG_ERR_ARG;
   if (dtype == FG_F32)
     moe_gate_up_generic_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, ldx, (const float*)wg, (const float*)wu,
-                                                                ldw, sorted, tiles, top, dim, hidden, (float*)act, lda);
+                                                                ldw, sorted, tiles, top, dim, hidden, (float*)act, lda, fn);
   else if (dtype == FG_BF16)
     moe_gate_up_generic_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)wg,
                                                                  (const bf16_t*)wu, ldw, sorted, tiles, top, dim, hidden,
-                                                                 (bf16_t*)act, lda);
+                                                                 (bf16_t*)act, lda, fn);
   else
     return FG_ERR_ARG;
   return fg_launch_status();
+}
+
+extern "C" int fg_moe_gate_up(const void* x, int ldx, const void* wg, const void* wu, int ldw, const int* sorted,
+                              const int* tiles, int max_tiles, int tile_rows, int top, int dim, int hidden, void* act,
+                              int lda, int dtype, int mfma, hipStream_t stream) {
+  return fg_moe_gate_up_act(x, ldx, wg, wu, ldw, sorted, tiles, max_tiles, tile_rows, top, dim, hidden, act, lda, dtype,
+                            mfma, FG_ACT_SILU, 0.f, 1.f, stream);
 }
 
 // act [n_pairs, lda] in the sorted order; wd [E, dim, ldw]; y fp32 [n_pairs, dim], row = pair.
@@ -609,8 +638,8 @@ extern "C" int fg_moe_down(const void* act, int lda, const void* wd, int ldw, co
     if ((tile_rows == 128 || tile_rows == 256) && hidden < 32) return FG_ERR_ARG;
     if (tile_rows == 128 || tile_rows == 256)
       return tile_rows == 128
-                 ? launch_moe_tiled<2, MT_DOWN>(act, lda, wd, nullptr, ldw, y, dim, sorted, tiles, max_tiles, 1, dim, hidden, stream)
-                 : launch_moe_tiled<4, MT_DOWN>(act, lda, wd, nullptr, ldw, y, dim, sorted, tiles, max_tiles, 1, dim, hidden, stream);
+                 ? launch_moe_tiled<2, MT_DOWN>(act, lda, wd, nullptr, ldw, y, dim, sorted, tiles, max_tiles, 1, dim, hidden, GatedAct{0, 0.f, 1.f}, stream)
+                 : launch_moe_tiled<4, MT_DOWN>(act, lda, wd, nullptr, ldw, y, dim, sorted, tiles, max_tiles, 1, dim, hidden, GatedAct{0, 0.f, 1.f}, stream);
     const long long items = (long long)max_tiles * ((dim + 15) / 16);
     const unsigned blocks = (unsigned)((items + 3) / 4);
 #define GO(MB)                                                                                                      \
@@ -640,35 +669,45 @@ extern "C" int fg_moe_down(const void* act, int lda, const void* wd, int ldw, co
 // ----------------------------------------------------------------- combine
 // out[t] = plus[t] + sum_j weight[t][j] * y[t * top + j]: the weighted sum first, j ascending, all fp32.
 // plus: rows of the activation dtype, or (n_plus > 0) fp32 partial sums plus[p * plus_stride + t * ldp + d],
-// whose sum, in order, is what is added.
+// whose sum, in order, is what is added.  plus_gate (fp32, one number a token at plus_gate[t * gate_stride]): the
+// rows of plus are multiplied by its sigmoid before they are added.
 template <class TP>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     const float* __restrict__ y, const float* __restrict__ weight, const TP* __restrict__ plus, int ldp, int n_plus,
-    size_t plus_stride, int top, int dim, float* __restrict__ out) {
+    size_t plus_stride, int top, int dim, float* __restrict__ out, const float* __restrict__ plus_gate, int gate_stride) {
   const int t = blockIdx.x;
+  const float pg = plus_gate ? 1.f / (1.f + expf(-plus_gate[(size_t)t * gate_stride])) : 1.f;
   for (int d = threadIdx.x; d < dim; d += 256) {
     float s = 0.f;
     for (int j = 0; j < top; ++j) s = fmaf(weight[(size_t)t * top + j], y[((size_t)t * top + j) * dim + d], s);
     if (plus) {
       float m = to_f<TP>(plus[(size_t)t * ldp + d]);
       for (int p = 1; p < n_plus; ++p) m += to_f<TP>(plus[p * plus_stride + (size_t)t * ldp + d]);
-      s = m + s;
+      s = (plus_gate ? m * pg : m) + s;
     }
     out[(size_t)t * dim + d] = s;
   }
 }
 
-extern "C" int fg_moe_combine(const float* y, const float* weight, const void* plus, int ldp, int plus_dtype, int n_plus,
-                              long long plus_stride, int n_tokens, int top, int dim, float* out, hipStream_t stream) {
+extern "C" int fg_moe_combine_gated(const float* y, const float* weight, const void* plus, int ldp, int plus_dtype,
+                                    int n_plus, long long plus_stride, int n_tokens, int top, int dim, float* out,
+                                    const float* plus_gate, int gate_stride, hipStream_t stream) {
   if (n_tokens <= 0) return FG_OK;
+  if (plus_gate && (!plus || gate_stride < 1)) return FG_ERR_ARG;
   if (top <= 0 || dim <= 0 || (plus && (ldp < dim || n_plus < 1)) || (n_plus > 1 && plus_dtype != FG_F32)) return FG_ERR_ARG;
   if (plus_dtype == FG_F32)
     moe_combine_kernel<float><<<n_tokens, 256, 0, stream>>>(y, weight, (const float*)plus, ldp, n_plus, (size_t)plus_stride,
-                                                            top, dim, out);
+                                                            top, dim, out, plus_gate, gate_stride);
   else if (plus_dtype == FG_BF16)
     moe_combine_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(y, weight, (const bf16_t*)plus, ldp, n_plus,
-                                                             (size_t)plus_stride, top, dim, out);
+                                                             (size_t)plus_stride, top, dim, out, plus_gate, gate_stride);
   else
     return FG_ERR_ARG;
   return fg_launch_status();
+}
+
+extern "C" int fg_moe_combine(const float* y, const float* weight, const void* plus, int ldp, int plus_dtype, int n_plus,
+                              long long plus_stride, int n_tokens, int top, int dim, float* out, hipStream_t stream) {
+  return fg_moe_combine_gated(y, weight, plus, ldp, plus_dtype, n_plus, plus_stride, n_tokens, top, dim, out, nullptr, 0,
+                              stream);
 }

@@ -529,10 +529,12 @@ extern "C" int fg_gelu_mul(const void* gu, void* out, int n_rows, int hidden, in
 // ------------------------------------------- act(g + b) * (u + b), any source dtype
 // The general form of the two kernels above: the rows may be fp32 (a product's un-rounded result) while
 // the result has the activation dtype, a bias per column of gu (fp32, in gu's interleaved order) is added
-// first, and the activation is SiLU (0), the tanh form of GELU (1) or ReLU (2).  All of it in fp32.
+// first, and the activation is SiLU (0), the tanh form of GELU (1) or ReLU (2), or (3) both halves are limited
+// first and the result is g * sigmoid(alpha g) * (u + 1) (GatedAct in common.h).  All of it in fp32.
 template <class TS, class TA>
 __global__ __launch_bounds__(ROWS_THREADS) void gated_mul_kernel(
-    const TS* __restrict__ gu, const float* __restrict__ bias, TA* __restrict__ out, int hidden, int act) {
+    const TS* __restrict__ gu, const float* __restrict__ bias, TA* __restrict__ out, int hidden, int act,
+    const GatedAct fn) {
   const TS* row = gu + (size_t)blockIdx.y * 2 * hidden;
   TA* o = out + (size_t)blockIdx.y * hidden;
   const int e = (blockIdx.x * ROWS_THREADS + threadIdx.x) * 8;
@@ -550,6 +552,10 @@ __global__ __launch_bounds__(ROWS_THREADS) void gated_mul_kernel(
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const float g = gv[i];
+      if (act == FG_ACT_LIMITED) {
+        r[i] = gated_act<false>(g, uv[i], fn);
+        continue;
+      }
       float a;
       if (act == 0) a = g / (1.f + expf(-g));
       else if (act == 1) a = 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
@@ -560,25 +566,33 @@ __global__ __launch_bounds__(ROWS_THREADS) void gated_mul_kernel(
   }
 }
 
-extern "C" int fg_gated_mul(const void* gu, const float* bias, void* out, int n_rows, int hidden, int act,
-                            int src_dtype, int act_dtype, hipStream_t stream) {
+extern "C" int fg_gated_mul_act(const void* gu, const float* bias, void* out, int n_rows, int hidden, int act,
+                                float limit, float alpha, int src_dtype, int act_dtype, hipStream_t stream) {
   if (n_rows <= 0) return FG_OK;
-  if (hidden <= 0 || hidden % 8 || n_rows > 65535 * 32 || act < 0 || act > 2) return FG_ERR_ARG;
+  if (hidden <= 0 || hidden % 8 || n_rows > 65535 * 32 || act < 0 || act > 3 || (act == 3 && !(limit > 0.f)))
+    return FG_ERR_ARG;
+  const GatedAct fn = {act, limit, alpha};
   for (int r0 = 0; r0 < n_rows; r0 += 65535) {
     const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
     const int per_block = ROWS_THREADS * 8;
     dim3 grid((hidden + per_block - 1) / per_block, nr);
     const size_t so = (size_t)r0 * 2 * hidden, oo = (size_t)r0 * hidden;
     if (src_dtype == FG_F32 && act_dtype == FG_F32)
-      gated_mul_kernel<float, float><<<grid, ROWS_THREADS, 0, stream>>>((const float*)gu + so, bias, (float*)out + oo, hidden, act);
+      gated_mul_kernel<float, float><<<grid, ROWS_THREADS, 0, stream>>>((const float*)gu + so, bias, (float*)out + oo, hidden, act, fn);
     else if (src_dtype == FG_F32 && act_dtype == FG_BF16)
-      gated_mul_kernel<float, bf16_t><<<grid, ROWS_THREADS, 0, stream>>>((const float*)gu + so, bias, (bf16_t*)out + oo, hidden, act);
+      gated_mul_kernel<float, bf16_t><<<grid, ROWS_THREADS, 0, stream>>>((const float*)gu + so, bias, (bf16_t*)out + oo, hidden, act, fn);
     else if (src_dtype == FG_BF16 && act_dtype == FG_BF16)
-      gated_mul_kernel<bf16_t, bf16_t><<<grid, ROWS_THREADS, 0, stream>>>((const bf16_t*)gu + so, bias, (bf16_t*)out + oo, hidden, act);
+      gated_mul_kernel<bf16_t, bf16_t><<<grid, ROWS_THREADS, 0, stream>>>((const bf16_t*)gu + so, bias, (bf16_t*)out + oo, hidden, act, fn);
     else
       return FG_ERR_ARG;
   }
   return fg_launch_status();
+}
+
+extern "C" int fg_gated_mul(const void* gu, const float* bias, void* out, int n_rows, int hidden, int act,
+                            int src_dtype, int act_dtype, hipStream_t stream) {
+  if (act < 0 || act > 2) return FG_ERR_ARG;
+  return fg_gated_mul_act(gu, bias, out, n_rows, hidden, act, 0.f, 1.f, src_dtype, act_dtype, stream);
 }
 
 // ------------------------------------------------------------- soft cap
@@ -592,5 +606,18 @@ extern "C" int fg_softcap(float* x, long long n, float cap, hipStream_t stream) 
   if (n <= 0) return FG_OK;
   if (!(cap > 0.f) || (n + ROWS_THREADS - 1) / ROWS_THREADS > 2147483647LL) return FG_ERR_ARG;
   softcap_kernel<<<(unsigned)((n + ROWS_THREADS - 1) / ROWS_THREADS), ROWS_THREADS, 0, stream>>>(x, (size_t)n, cap);
+  return fg_launch_status();
+}
+
+// x *= factor in place on fp32 (logits that a model multiplies by a constant).
+__global__ __launch_bounds__(ROWS_THREADS) void scale_kernel(float* __restrict__ x, size_t n, float factor) {
+  const size_t i = (size_t)blockIdx.x * ROWS_THREADS + threadIdx.x;
+  if (i < n) x[i] *= factor;
+}
+
+extern "C" int fg_scale(float* x, long long n, float factor, hipStream_t stream) {
+  if (n <= 0) return FG_OK;
+  if ((n + ROWS_THREADS - 1) / ROWS_THREADS > 2147483647LL) return FG_ERR_ARG;
+  scale_kernel<<<(unsigned)((n + ROWS_THREADS - 1) / ROWS_THREADS), ROWS_THREADS, 0, stream>>>(x, (size_t)n, factor);
   return fg_launch_status();
 }

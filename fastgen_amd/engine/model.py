@@ -18,7 +18,7 @@ import torch
 
 from ..config import ModelLayout, PartSpec, get_architecture, read_config_json
 from ..kernels.linear import StreamedMatrix, packing, packing_fits
-from ..kernels.ops import PostNormed, ScaledRows, post_add_rmsnorm
+from ..kernels.ops import PostNormed, ScaledRows, post_add_rmsnorm, streams_spread
 from ..parts import LayerStore, PagedNeed, StateNeed, TensorSpec, build_part
 from ..parts.base import MATRIX
 from ..weights.source import RandomSource, SafetensorsSource, TensorSource, check_against_specs
@@ -54,9 +54,13 @@ def build_parts(layout: ModelLayout) -> ModelParts:
         n2 = build_part("norm", ls.ffn_norm) if ls.ffn_norm is not None else None
         extra = {name: build_part("norm", spec) for name, spec in ls.extra_norms.items()}
         # an arrangement that asks for no further norms is built from the four parts alone
-        blocks.append(build_part("arrangement", PartSpec(ls.arrangement), mixer, ffn, n1, n2, *([extra] if extra else [])))
+        block = build_part("arrangement", ls.arrangement_spec or PartSpec(ls.arrangement), mixer, ffn, n1, n2,
+                           *([extra] if extra else []))
+        blocks.append(block)
         mixers.append(mixer)
         parts += [p for p in (mixer, ffn, n1, n2, *extra.values()) if p is not None]
+        if hasattr(block, "tensor_specs"):  # an arrangement with tensors of its own
+            parts.append(block)
     injections = [build_part("injection", spec) for spec in layout.injections]
     final_norm = build_part("norm", layout.final_norm)
     head = build_part("head", layout.head)
@@ -174,6 +178,8 @@ class Model:
         if not self.loaded:
             raise RuntimeError("the model has no weights yet")
         h = self.parts.embed.forward(ctx.tokens, ctx)
+        if self.layout.streams:
+            h = streams_spread(h, self.layout.streams)  # [S, T, dim]: the blocks and the last norm know
         injections = self.parts.injections
         # the embedding's output as it was, for injections that add it again (h itself moves on)
         embedded = h.clone() if any(p.needs_embedding for p in injections) else None

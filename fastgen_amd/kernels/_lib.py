@@ -49,6 +49,7 @@ LIBRARIES: Dict[str, str] = {
     "recurrence": "recurrence.hip",
     "selective_scan": "selective_scan.hip",
     "sigmoid_attention": "sigmoid_attention.hip",
+    "streams": "streams.hip",
 }
 
 # libraries compiled once per value of a macro: name -> (source, macro, values that build_all compiles,

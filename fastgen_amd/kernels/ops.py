@@ -314,6 +314,14 @@ def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
 
 
 # ------------------------------------------------------------ rope + kv write
+def scale_logits(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """``x *= factor`` in place on contiguous fp32."""
+    _gpu(x)
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "x must be contiguous float32")
+    _check(_lib.load("rows").fg_scale(_ptr(x), ctypes.c_longlong(x.numel()), ctypes.c_float(factor), _stream(x)), "scale_logits")
+    return x
+
+
 def rope_table(positions: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
     """``[T, n_freqs, 2]`` fp32: cos and sin of ``float(pos) * freqs[i]``, for all
     layers of a step that rotate with the same frequencies."""
@@ -388,7 +396,9 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
     ``q`` is ``[T, >= H*hd]`` (the first ``H*hd`` columns are the query heads;
     it may be a qkv buffer), ``out`` is ``[T, H*hd]``.  ``forward.py:176-258``.
     ``sinks``: fp32 ``[H]``; head ``h``'s softmax has one more term ``exp(sinks[h])`` in its
-    denominator, which brings no value.
+    denominator, which brings no value.  ``window`` > 0: a token at position ``p`` sees the keys
+    ``p - window + 1 .. p``; ``window`` < 0: the keys up to ``p`` of its own block of ``-window`` positions,
+    blocks counted from position 0 of the sequence (:func:`block_mask`); 0: every key up to ``p``.
     """
     _gpu(q, out, k_pages, v_pages, block_table, seq_of_token, positions, sinks)
     _sinks_ok(sinks, n_heads)
@@ -413,6 +423,12 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
         ctypes.c_float(scale), int(window or 0), _ptr(sinks), _code(q), _stream(q))
     _check(st, "paged_attention_general")
     return out
+
+
+def block_mask(size: Optional[int]) -> int:
+    """The ``window`` argument of the attention functions for a mask of blocks of ``size`` positions: a token
+    sees the keys before it (and itself) inside its own block, blocks counted from position 0."""
+    return -int(size) if size else 0
 
 
 MFMA_MAX_HEAD_DIM = 256
@@ -1004,7 +1020,7 @@ MOE_TILE_ROWS = (16, 32, 64, 128, 256)  # rows of one expert that a tile of the 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int,
               sigmoid_scores: bool = False, correction: Optional[torch.Tensor] = None, n_groups: int = 1,
-              keep_groups: int = 1, weight_scale: float = 1.0):
+              keep_groups: int = 1, weight_scale: float = 1.0, softmax_scores: bool = False, n_extra: int = 0):
     """Per row of ``x [T, dim]``: fp32 logits ``x router^T + bias`` (``router`` fp32 ``[E, dim]``), the
     ``top`` largest (ties: the lower expert), and the softmax over those.  Returns int32 ``[T, top]``
     experts and fp32 ``[T, top]`` weights, the largest logit first.
@@ -1013,27 +1029,35 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     ``correction`` (fp32 ``[E]`` or None) among the experts of the ``keep_groups`` best of ``n_groups`` equal
     groups of neighbours (a group ranks by the sum of its two largest choice scores; ties: the lower group);
     the weights are the chosen experts' scores, without the correction, divided by their sum (+ 1e-20)
-    and multiplied by ``weight_scale``."""
+    and multiplied by ``weight_scale``.  ``softmax_scores``: the same with the softmax of the logits over all
+    experts as the scores.
+
+    ``n_extra``: ``router`` has that many rows behind the experts'; their logits (without bias) take no part in
+    the choice and are returned as a third result, fp32 ``[T, n_extra]`` (the gate of a shared expert, say)."""
     _gpu(x, router, bias, correction)
     _need(x.dim() == 2 and x.stride(1) == 1 and x.data_ptr() % 16 == 0, "x must be [T, dim] with unit column stride")
     T, dim = x.shape
-    E = router.shape[0]
-    _need(router.dtype == torch.float32 and router.shape == (E, dim) and router.is_contiguous(),
-          "router must be contiguous float32 [E, dim]")
+    E = router.shape[0] - int(n_extra)
+    _need(n_extra >= 0 and E >= 1 and not (sigmoid_scores and softmax_scores), "n_extra rows behind at least one expert; one way of scoring")
+    _need(router.dtype == torch.float32 and router.shape == (E + n_extra, dim) and router.is_contiguous(),
+          "router must be contiguous float32 [E + n_extra, dim]")
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.shape == (E,) and bias.is_contiguous(), "bias must be float32 [E]")
     _need(1 <= top <= E, f"top={top} must be between 1 and the {E} experts")
     choice = torch.empty((T, top), dtype=torch.int32, device=x.device)
     weight = torch.empty((T, top), dtype=torch.float32, device=x.device)
     _f32_vec(correction, E, "correction")
-    _need(sigmoid_scores or (correction is None and n_groups == 1), "correction and groups go with sigmoid scores")
+    scored = sigmoid_scores or softmax_scores
+    _need(scored or (correction is None and n_groups == 1), "correction and groups go with sigmoid or softmax scores")
+    extra = torch.empty((T, n_extra), dtype=torch.float32, device=x.device) if n_extra else None
     _need(n_groups >= 1 and E % n_groups == 0 and 1 <= keep_groups <= n_groups and top <= keep_groups * (E // n_groups),
           f"{n_groups} groups of which {keep_groups} stay do not fit {E} experts and top={top}")
     st = _lib.load("moe").fg_moe_route_mode(_ptr(x), x.stride(0), _code(x), _ptr(router), _ptr(bias), T, dim, E, top,
-                                            _ptr(choice), _ptr(weight), int(bool(sigmoid_scores)), _ptr(correction),
-                                            int(n_groups), int(keep_groups), ctypes.c_float(weight_scale), _stream(x))
+                                            _ptr(choice), _ptr(weight), 2 if softmax_scores else int(bool(sigmoid_scores)),
+                                            _ptr(correction), int(n_groups), int(keep_groups),
+                                            ctypes.c_float(weight_scale), int(n_extra), _ptr(extra), _stream(x))
     _check(st, "moe_route")
-    return choice, weight
+    return (choice, weight, extra) if n_extra else (choice, weight)
 
 
 def moe_max_tiles(n_pairs: int, n_experts: int, tile_rows: int) -> int:
@@ -1064,8 +1088,10 @@ def _moe_mfma_ok(x: torch.Tensor, *weights: torch.Tensor) -> bool:
 
 
 def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, sorted_: torch.Tensor, tiles: torch.Tensor,
-                top: int, tile_rows: int) -> torch.Tensor:
+                top: int, tile_rows: int, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
     """``silu(x_t W_gate[e]^T) * (x_t W_up[e]^T)`` for every pair, in the sorted order: ``[T * top, hidden]``.
+    With ``limit`` > 0 the activation is the limited one: ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``,
+    ``g * sigmoid(alpha * g) * (u + 1)``.
     ``w_gate``, ``w_up``: ``[E, hidden, dim]`` of ``x``'s dtype.  bfloat16 with sizes in multiples of 8
     runs on the matrix cores; everything else the fp32-FMA kernel (tiles of 16 rows only)."""
     _gpu(x, w_gate, w_up, sorted_, tiles)
@@ -1079,9 +1105,10 @@ def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, sorte
     mfma = _moe_mfma_ok(x, w_gate) and hidden % 8 == 0
     _need(tile_rows in MOE_TILE_ROWS and (mfma or tile_rows == 16), "tile_rows does not fit the kernel")
     act = torch.empty((sorted_.numel(), hidden), dtype=x.dtype, device=x.device)
-    st = _lib.load("moe").fg_moe_gate_up(_ptr(x), x.stride(0), _ptr(w_gate), _ptr(w_up), dim, _ptr(sorted_), _ptr(tiles),
-                                         tiles.shape[0], tile_rows, top, dim, hidden, _ptr(act), hidden, _code(x), int(mfma),
-                                         _stream(x))
+    st = _lib.load("moe").fg_moe_gate_up_act(_ptr(x), x.stride(0), _ptr(w_gate), _ptr(w_up), dim, _ptr(sorted_), _ptr(tiles),
+                                             tiles.shape[0], tile_rows, top, dim, hidden, _ptr(act), hidden, _code(x),
+                                             int(mfma), ACT_LIMITED if limit > 0 else 0, ctypes.c_float(limit),
+                                             ctypes.c_float(alpha), _stream(x))
     _check(st, "moe_gate_up")
     return act
 
@@ -1107,11 +1134,16 @@ def moe_down(act: torch.Tensor, w_down: torch.Tensor, sorted_: torch.Tensor, til
     return y
 
 
-def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tensor] = None) -> torch.Tensor:
+def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tensor] = None,
+                plus_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp32 ``[1, T, dim]``: ``plus[t] + sum_j weight[t, j] * y[t * top + j]``, the weighted sum first, ``j``
     ascending.  ``plus``: ``[T, dim]`` rows of any supported dtype, fp32 ``[S, T, dim]`` partial sums (a
-    product whose k range was cut; summed in order), or None."""
-    _gpu(y, weight, plus)
+    product whose k range was cut; summed in order), or None.  ``plus_gate``: fp32 ``[T]`` (any stride): the rows
+    of ``plus`` are multiplied by ``sigmoid(plus_gate[t])`` before they are added."""
+    _gpu(y, weight, plus, plus_gate)
+    if plus_gate is not None:
+        _need(plus is not None and plus_gate.dtype == torch.float32 and plus_gate.dim() == 1
+              and plus_gate.shape[0] == weight.shape[0] and plus_gate.stride(0) >= 1, "plus_gate must be float32 [T], with plus")
     T, top = weight.shape
     _need(y.dtype == torch.float32 and y.dim() == 2 and y.shape[0] == T * top and y.is_contiguous()
           and weight.dtype == torch.float32 and weight.is_contiguous(), "y float32 [T * top, dim], weight float32 [T, top]")
@@ -1125,8 +1157,9 @@ def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tens
         _need(plus.shape == (T, dim) and plus.stride(1) == 1, "plus must be [T, dim]")
         ldp, n_plus = plus.stride(0), 1
     out = torch.empty((1, T, dim), dtype=torch.float32, device=y.device)
-    st = _lib.load("moe").fg_moe_combine(_ptr(y), _ptr(weight), _ptr(plus), ldp, _code(plus) if plus is not None else F32,
-                                         n_plus, ctypes.c_longlong(stride), T, top, dim, _ptr(out), _stream(y))
+    st = _lib.load("moe").fg_moe_combine_gated(_ptr(y), _ptr(weight), _ptr(plus), ldp, _code(plus) if plus is not None else F32,
+                                               n_plus, ctypes.c_longlong(stride), T, top, dim, _ptr(out), _ptr(plus_gate),
+                                               plus_gate.stride(0) if plus_gate is not None else 0, _stream(y))
     _check(st, "moe_combine")
     return out
 
@@ -1300,6 +1333,117 @@ def head_norm_gate(x: torch.Tensor, weight: torch.Tensor, eps: float, gate: torc
 
 
 # ---------------------------------------------------------------- recurrence
+def head_diff_norm(att: torch.Tensor, head_width: int, out: torch.Tensor, n_heads: int, group: int, v_width: int,
+                   lam: float, eps: float, out_scale: float) -> torch.Tensor:
+    """Two attention maps a head over one value: ``out[t, h, :] = n(a1 - lam * a2) * out_scale`` with ``n`` the
+    division by the root mean square over the head's ``v_width`` values (``eps`` inside the root).  ``att [T, 2 H *
+    head_width]`` holds, per key/value group of ``group`` query heads, the first maps' outputs of the group's heads
+    and then the second maps' (each ``head_width`` wide, the first ``v_width`` columns count); ``out [T, H *
+    v_width]`` of the same dtype."""
+    _gpu(att, out)
+    T = att.shape[0]
+    _need(att.dim() == 2 and att.stride(1) == 1 and att.shape[1] >= 2 * n_heads * head_width and head_width >= v_width > 0,
+          "att must be [T, >= 2 H * head_width] with heads at least v_width wide")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == T and out.shape[1] >= n_heads * v_width
+          and out.dtype == att.dtype, "out must be [T, >= H * v_width] of att's dtype")
+    _need(group >= 1 and n_heads % group == 0 and v_width <= 1024, "heads in whole groups, of at most 1024 values")
+    st = _lib.load("heads").fg_head_diff_norm(_ptr(att), att.stride(0), head_width, _ptr(out), out.stride(0), T, n_heads,
+                                              group, v_width, ctypes.c_float(lam), ctypes.c_float(eps),
+                                              ctypes.c_float(out_scale), _code(att), _stream(att))
+    _check(st, "head_diff_norm")
+    return out
+
+
+# ------------------------------------------------------- several residual streams
+@dataclass
+class StreamUpdate:
+    """A sublayer's output on its way into several residual streams: ``rows`` (``[T, dim]`` of the activation
+    dtype or fp32 ``[P, T, dim]`` partial sums) goes into stream ``t`` times ``out[t]`` while the streams are
+    mixed by ``mix [S, S]`` (from-stream by to-stream): ``X'[t] = sum_s mix[s, t] X[s] + out[t] rows``.  What norms
+    the streams next applies it (:func:`streams_step`)."""
+
+    rows: torch.Tensor
+    mix: torch.Tensor  # fp32 [S, S]
+    out: torch.Tensor  # fp32 [S]
+
+
+class _StreamArgs(ctypes.Structure):
+    _fields_ = [("x", ctypes.c_void_p), ("delta", ctypes.c_void_p), ("parts", ctypes.c_void_p), ("n_parts", ctypes.c_int),
+                ("part_stride", ctypes.c_longlong), ("mix", ctypes.c_void_p), ("out_w", ctypes.c_void_p),
+                ("in_w", ctypes.c_void_p), ("norm_w", ctypes.c_void_p), ("out", ctypes.c_void_p), ("u_out", ctypes.c_void_p),
+                ("rows", ctypes.c_void_p), ("n_streams", ctypes.c_int), ("n_tokens", ctypes.c_int), ("dim", ctypes.c_int),
+                ("eps", ctypes.c_float)]
+
+
+STREAMS_MAX = 8
+
+
+def streams_spread(h: torch.Tensor, n_streams: int) -> torch.Tensor:
+    """fp32 ``[S, T, dim]``: ``h [T, dim]`` copied into every one of ``n_streams`` residual streams."""
+    _gpu(h)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous() and 1 <= n_streams <= STREAMS_MAX,
+          f"h must be contiguous float32 [T, dim], at most {STREAMS_MAX} streams")
+    x = torch.empty((n_streams, *h.shape), dtype=torch.float32, device=h.device)
+    _check(_lib.load("streams").fg_streams_spread(_ptr(h), _ptr(x), ctypes.c_longlong(h.numel()), n_streams, _stream(h)),
+           "streams_spread")
+    return x
+
+
+def streams_step(x: torch.Tensor, update: Optional[StreamUpdate], in_weights: Optional[torch.Tensor],
+                 norm_weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
+                 rows: Optional[torch.Tensor] = None, u_out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """On the residual streams ``x`` (fp32 ``[S, T, dim]``), all in fp32: apply ``update`` (in place; None: nothing
+    is pending), form ``u = sum_s in_weights[s] x[s]`` (``in_weights`` fp32 ``[S]``; None: the plain sum), and store
+    ``out = rmsnorm(u) * norm_weight`` (``[T, dim]``, rounded once to its dtype; without ``norm_weight``: ``u`` itself)
+    and/or ``u_out = u`` in fp32.  With ``rows`` only those tokens are computed, into consecutive rows, and ``x`` is
+    left as it was."""
+    _gpu(x, in_weights, norm_weight, out, rows, u_out, *(() if update is None else (update.rows, update.mix, update.out)))
+    _need(x.dtype == torch.float32 and x.dim() == 3 and x.is_contiguous() and 1 <= x.shape[0] <= STREAMS_MAX,
+          f"x must be contiguous float32 [S, T, dim], at most {STREAMS_MAX} streams")
+    S, T, dim = x.shape
+    _need(dim <= 8192, "rows of at most 8192 elements")
+    n_rows = T if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, "rows")
+    a = _StreamArgs()
+    a.x, a.n_streams, a.n_tokens, a.dim, a.eps = x.data_ptr(), S, T, dim, eps
+    act = out.dtype if out is not None else None
+    if update is not None:
+        _f32_vec(update.mix, S * S, "update.mix")
+        _f32_vec(update.out, S, "update.out")
+        _need(update.mix.numel() == S * S and update.out.numel() == S, "update.mix must be [S, S], update.out [S]")
+        d = update.rows
+        if d.dim() == 3:
+            _need(d.dtype == torch.float32 and d.shape[1:] == (T, dim) and d.stride(2) == 1 and d.stride(1) == dim,
+                  "partial sums must be float32 [P, T, dim] with contiguous rows")
+            a.parts, a.n_parts, a.part_stride = d.data_ptr(), d.shape[0], d.stride(0)
+        else:
+            _need(d.shape == (T, dim) and d.is_contiguous() and (act is None or d.dtype == act),
+                  "the update's rows must be contiguous [T, dim] of out's dtype")
+            a.delta, act = d.data_ptr(), d.dtype
+        a.mix, a.out_w = update.mix.data_ptr(), update.out.data_ptr()
+    _need(update is not None or out is not None or u_out is not None, "nothing to apply and nothing to store")
+    if in_weights is not None:
+        _f32_vec(in_weights, S, "in_weights")
+        a.in_w = in_weights.data_ptr()
+    if norm_weight is not None:
+        _need(norm_weight.shape == (dim,) and norm_weight.is_contiguous() and out is not None, "norm_weight must be [dim], with out")
+        a.norm_w = norm_weight.data_ptr()
+    if out is not None:
+        _need(out.is_contiguous() and out.shape == (n_rows, dim), "out must be contiguous [rows, dim]")
+        a.out = out.data_ptr()
+    if u_out is not None:
+        _need(u_out.is_contiguous() and u_out.shape == (n_rows, dim) and u_out.dtype == torch.float32,
+              "u_out must be contiguous float32 [rows, dim]")
+        a.u_out = u_out.data_ptr()
+    if rows is not None:
+        a.rows = rows.data_ptr()
+    st = _lib.load("streams").fg_streams_step_rows(ctypes.byref(a), n_rows, _DTYPE_CODE[act or torch.float32],
+                                                   _code(norm_weight) if norm_weight is not None else F32, _stream(x))
+    _check(st, "streams_step")
+    return out if out is not None else u_out
+
+
 class _ScanArgs(ctypes.Structure):
     _fields_ = [("qkv", ctypes.c_void_p), ("row_stride", ctypes.c_int), ("q_col", ctypes.c_int), ("k_col", ctypes.c_int),
                 ("v_col", ctypes.c_int), ("decay", ctypes.c_void_p), ("decay_stride", ctypes.c_int),
@@ -1382,14 +1526,16 @@ def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.T
 
 
 # ----------------------------------------------------- gated activation, general
-_ACT_CODE = {"silu": 0, "gelu_tanh": 1, "relu": 2}
+ACT_LIMITED = 3
+_ACT_CODE = {"silu": 0, "gelu_tanh": 1, "relu": 2, "limited": ACT_LIMITED}
 
 
 def gated_mul(gate_up: torch.Tensor, bias: Optional[torch.Tensor], activation: str, out_dtype: torch.dtype,
-              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+              out: Optional[torch.Tensor] = None, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
     """``act(gate + b) * (up + b)`` for ``gate_up [T, 2 * hidden]`` as :func:`interleave_gate_up` orders it (fp32, or
     ``out_dtype``), ``bias`` fp32 ``[2 * hidden]`` in the same order (or None), ``activation`` one of ``silu``,
-    ``gelu_tanh``, ``relu``.  All of it in fp32, one rounding to ``out_dtype``."""
+    ``gelu_tanh``, ``relu``, or ``limited``: ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``,
+    ``g * sigmoid(alpha * g) * (u + 1)``.  All of it in fp32, one rounding to ``out_dtype``."""
     _gpu(gate_up, bias, out)
     _need(activation in _ACT_CODE, f"activation {activation!r} is not supported ({sorted(_ACT_CODE)})")
     _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 16 == 0,
@@ -1400,8 +1546,10 @@ def gated_mul(gate_up: torch.Tensor, bias: Optional[torch.Tensor], activation: s
     if out is None:
         out = torch.empty((T, hidden), dtype=out_dtype, device=gate_up.device)
     _need(out.shape == (T, hidden) and out.is_contiguous() and out.dtype == out_dtype, "out must be contiguous [T, hidden]")
-    st = _lib.load("rows").fg_gated_mul(_ptr(gate_up), _ptr(bias), _ptr(out), T, hidden, _ACT_CODE[activation],
-                                        _code(gate_up), _code(out), _stream(out))
+    _need(activation != "limited" or limit > 0, "the limited activation needs a positive limit")
+    st = _lib.load("rows").fg_gated_mul_act(_ptr(gate_up), _ptr(bias), _ptr(out), T, hidden, _ACT_CODE[activation],
+                                            ctypes.c_float(limit), ctypes.c_float(alpha), _code(gate_up), _code(out),
+                                            _stream(out))
     _check(st, "gated_mul")
     return out
 

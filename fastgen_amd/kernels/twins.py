@@ -157,6 +157,10 @@ def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
     return x
 
 
+def scale_logits(x: torch.Tensor, factor: float) -> torch.Tensor:
+    return x.mul_(factor)
+
+
 def rope_table(positions: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
     """fp32 ``[T, len(freqs), 2]``: cos and sin of ``position * frequency``."""
     ang = positions.to(torch.float32)[:, None] * freqs.float()[None, :]
@@ -219,7 +223,8 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
                             block_table: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
                             n_heads: int, scale: float, window: int = 0,
                             sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Token ``t`` of sequence ``b`` at position ``p`` attends keys ``0..p`` (``p-window+1..p`` with a window)
+    """Token ``t`` of sequence ``b`` at position ``p`` attends keys ``0..p`` (``p-window+1..p`` with a window; with a
+    negative one the keys up to ``p`` of its block of ``-window`` positions, blocks counted from 0)
     of its sequence, read through ``block_table[b]``; query head ``h`` reads kv head ``h // (H / KV)``;
     softmax of ``scale * q.k`` in fp32 (``fastgen/forward.py:176-258``).  With ``sinks`` head ``h``'s softmax runs
     over one more score, ``sinks[h]`` as it is, whose weight meets no value."""
@@ -229,7 +234,7 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
         b, p = int(seq_of_token[t]), int(positions[t])
         k = _gather_kv(k_pages, unpack_k, block_table[b], p + 1)
         v = _gather_kv(v_pages, unpack_v, block_table[b], p + 1)
-        lo = max(0, p - window + 1) if window else 0
+        lo = max(0, p - window + 1) if window > 0 else (p - p % -window if window < 0 else 0)
         qt = q[t, : n_heads * hd].float().view(n_heads, hd)
         for h in range(n_heads):
             s = (k[lo:, h // G] @ qt[h]) * scale
@@ -371,16 +376,21 @@ def gemm_skinny_qkv(x, wqkv, table: Optional[torch.Tensor], slots: torch.Tensor,
 # ------------------------------------------------------------- routed experts
 def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int,
               sigmoid_scores: bool = False, correction: Optional[torch.Tensor] = None, n_groups: int = 1,
-              keep_groups: int = 1, weight_scale: float = 1.0):
+              keep_groups: int = 1, weight_scale: float = 1.0, softmax_scores: bool = False, n_extra: int = 0):
     """The ``top`` experts with the largest fp32 logits ``x router^T + bias`` (largest first; of equal
     logits the lower expert) and the softmax over those logits alone.  With ``sigmoid_scores``: scores
     ``sigmoid(logit)``; chosen by score plus ``correction`` inside the ``keep_groups`` groups (of ``n_groups``) whose two
-    largest choice scores sum highest; weights: the chosen scores over their sum (+ 1e-20), times ``weight_scale``."""
-    z = x.float() @ router.T + (bias if bias is not None else 0.0)
-    if not sigmoid_scores:
+    largest choice scores sum highest; weights: the chosen scores over their sum (+ 1e-20), times ``weight_scale``.
+    ``softmax_scores``: the same with scores ``softmax(logits)`` over all experts.  The last ``n_extra`` rows of
+    ``router`` are no experts: their logits come back as a third result."""
+    z = x.float() @ router.T
+    E = router.shape[0] - n_extra
+    z, extra = z[:, :E] + (bias if bias is not None else 0.0), z[:, E:]
+    more = (extra,) if n_extra else ()
+    if not (sigmoid_scores or softmax_scores):
         val, idx = torch.sort(z, dim=-1, descending=True, stable=True)
-        return idx[:, :top].to(torch.int32), torch.softmax(val[:, :top], dim=-1)
-    score = torch.sigmoid(z)
+        return (idx[:, :top].to(torch.int32), torch.softmax(val[:, :top], dim=-1), *more)
+    score = torch.softmax(z, dim=-1) if softmax_scores else torch.sigmoid(z)
     choice = score + (correction if correction is not None else 0.0)
     T, E = choice.shape
     if n_groups > 1 and keep_groups < n_groups:
@@ -391,7 +401,7 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
         choice = choice.masked_fill(lost[:, :, None].expand(T, n_groups, per).reshape(T, E), float("-inf"))
     idx = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
     w = score.gather(1, idx)
-    return idx.to(torch.int32), w / (w.sum(-1, keepdim=True) + 1e-20) * weight_scale
+    return (idx.to(torch.int32), w / (w.sum(-1, keepdim=True) + 1e-20) * weight_scale, *more)
 
 
 def moe_max_tiles(n_pairs: int, n_experts: int, tile_rows: int) -> int:
@@ -422,13 +432,19 @@ def _expert_of_place(sorted_: torch.Tensor, tiles: torch.Tensor) -> torch.Tensor
 
 
 def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, sorted_: torch.Tensor, tiles: torch.Tensor,
-                top: int, tile_rows: int) -> torch.Tensor:
-    """``silu(x_t w_gate[e]^T) * (x_t w_up[e]^T)`` for the pair at every sorted place, ``e`` its expert."""
+                top: int, tile_rows: int, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+    """``silu(x_t w_gate[e]^T) * (x_t w_up[e]^T)`` for the pair at every sorted place, ``e`` its expert; with a
+    ``limit``: ``g * sigmoid(alpha g) * (u + 1)`` of ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``."""
     expert = _expert_of_place(sorted_, tiles)
     rows = x[sorted_.long() // top].float()
     g = torch.einsum("pk,pfk->pf", rows, w_gate[expert].float())
     u = torch.einsum("pk,pfk->pf", rows, w_up[expert].float())
-    return (g * torch.sigmoid(g) * u).to(x.dtype)
+    return (_limited(g, u, limit, alpha) if limit > 0 else g * torch.sigmoid(g) * u).to(x.dtype)
+
+
+def _limited(g: torch.Tensor, u: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    g, u = g.clamp(max=limit), u.clamp(min=-limit, max=limit)
+    return g * torch.sigmoid(alpha * g) * (u + 1.0)
 
 
 def moe_down(act: torch.Tensor, w_down: torch.Tensor, sorted_: torch.Tensor, tiles: torch.Tensor,
@@ -440,12 +456,14 @@ def moe_down(act: torch.Tensor, w_down: torch.Tensor, sorted_: torch.Tensor, til
     return y
 
 
-def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """fp32 ``[1, T, dim]``: ``plus[t] + sum_j weight[t, j] * y[t * top + j]``."""
+def moe_combine(y: torch.Tensor, weight: torch.Tensor, plus: Optional[torch.Tensor] = None,
+                plus_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 ``[1, T, dim]``: ``plus[t] (* sigmoid(plus_gate[t])) + sum_j weight[t, j] * y[t * top + j]``."""
     T, top = weight.shape
     out = (weight[:, :, None] * y.view(T, top, -1)).sum(1)
     if plus is not None:
-        out = (plus.sum(0) if plus.dim() == 3 else plus.float()) + out
+        p = plus.sum(0) if plus.dim() == 3 else plus.float()
+        out = (p * torch.sigmoid(plus_gate.float())[:, None] if plus_gate is not None else p) + out
     return out[None]
 
 
@@ -581,13 +599,14 @@ def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.T
 
 # ----------------------------------------------------- gated activation, general
 def gated_mul(gate_up: torch.Tensor, bias: Optional[torch.Tensor], activation: str, out_dtype: torch.dtype,
-              out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``act(gate + b) * (up + b)`` for rows interleaved in groups of 8 (gate, up); ``silu``, ``gelu_tanh`` or ``relu``."""
+              out: Optional[torch.Tensor] = None, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+    """``act(gate + b) * (up + b)`` for rows interleaved in groups of 8 (gate, up); ``silu``, ``gelu_tanh``, ``relu``, or
+    ``limited`` (``g * sigmoid(alpha g) * (u + 1)`` of the halves limited first)."""
     y = gate_up.float() + (bias.float() if bias is not None else 0.0)
     y = y.reshape(y.shape[0], -1, 2, 8)
     g, u = y[:, :, 0].reshape(y.shape[0], -1), y[:, :, 1].reshape(y.shape[0], -1)
     a = torch.relu(g) if activation == "relu" else _gelu_tanh(g) if activation == "gelu_tanh" else g * torch.sigmoid(g)
-    r = (a * u).to(out_dtype)
+    r = (_limited(g, u, limit, alpha) if activation == "limited" else a * u).to(out_dtype)
     if out is None:
         return r
     out.copy_(r)
@@ -675,3 +694,43 @@ def sigmoid_attention(q: torch.Tensor, head_dim: int, out: torch.Tensor, v_head_
             o = o * torch.sigmoid(gate[t, :H].float())[:, None]
         out[t, : H * e] = o.reshape(-1).to(out.dtype)
     return out
+
+
+# ------------------------------------------------------- two maps a head, several streams
+def head_diff_norm(att: torch.Tensor, head_width: int, out: torch.Tensor, n_heads: int, group: int, v_width: int,
+                   lam: float, eps: float, out_scale: float) -> torch.Tensor:
+    """``out[t, h] = o / sqrt(mean(o^2) + eps) * out_scale`` with ``o = a1 - lam a2``; per key/value group ``att`` holds the
+    first maps' outputs of the group's heads, then the second maps'."""
+    T = att.shape[0]
+    a = att[:, : 2 * n_heads * head_width].float().view(T, n_heads // group, 2, group, head_width)[..., :v_width]
+    o = (a[:, :, 0] - lam * a[:, :, 1]).reshape(T, n_heads, v_width)
+    o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * out_scale
+    out[:, : n_heads * v_width] = o.reshape(T, -1).to(out.dtype)
+    return out
+
+
+def streams_spread(h: torch.Tensor, n_streams: int) -> torch.Tensor:
+    return h[None].repeat(n_streams, 1, 1)
+
+
+def streams_step(x: torch.Tensor, update, in_weights: Optional[torch.Tensor], norm_weight: Optional[torch.Tensor],
+                 eps: float, out: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
+                 u_out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``x' [t] = sum_s mix[s, t] x[s] + out_w[t] y`` (if an update is pending), ``u = sum_s in_weights[s] x'[s]``,
+    ``out = rmsnorm(u) * norm_weight`` (or ``u``), ``u_out = u``; with ``rows`` only those tokens, ``x`` untouched."""
+    S = x.shape[0]
+    new = x
+    if update is not None:
+        y = update.rows.sum(0) if update.rows.dim() == 3 else update.rows.float()
+        new = torch.einsum("sr,std->rtd", update.mix.view(S, S), x) + update.out.view(S, 1, 1) * y[None]
+        if rows is None:
+            x.copy_(new)
+    u = new.sum(0) if in_weights is None else torch.einsum("s,std->td", in_weights, new)
+    if rows is not None:
+        u = u[rows.long()]
+    if u_out is not None:
+        u_out.copy_(u)
+    if out is not None:
+        n = u if norm_weight is None else u / torch.sqrt((u * u).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        out.copy_(n.to(out.dtype))
+    return out if out is not None else u_out

@@ -18,8 +18,8 @@ from .base import (
     registered_parts,
     unregister_part,
 )
-from . import (attention, block, embedding, feed_forward, injection, latent_attention, linear_attention, moe, norm,  # noqa: F401
-               position, selective_scan, sigmoid_attention)  # register the built-in parts
+from . import (attention, block, differential_attention, embedding, feed_forward, injection, latent_attention,  # noqa: F401
+               linear_attention, moe, norm, position, selective_scan, sigmoid_attention)  # register the built-in parts
 
 __all__ = [
     "MATRIX", "TABLE_INT", "VECTOR", "FeedForward", "Injection", "LayerStore", "Mixer", "Norm", "PagedNeed", "Part",

@@ -9,7 +9,7 @@ import torch
 
 from ..kernels import ops
 from ..kernels.ops import ScaledRows
-from .base import FeedForward, LayerStore, Mixer, Norm, register_part
+from .base import VECTOR, FeedForward, LayerStore, Mixer, Norm, Part, TensorSpec, register_part
 
 
 def _no_output_bias(ffn, arrangement: str) -> None:
@@ -164,3 +164,70 @@ class NormBehindBlock:
 
 
 register_part("arrangement", "norm_behind", lambda spec, *parts: NormBehindBlock(*parts))
+
+
+class HyperConnectionBlock(Part):
+    """Several residual streams side by side.  The model keeps ``streams`` copies ``X[0..S-1]`` of the residual
+    stream (fp32 ``[S, T, dim]``; all equal the embedding's output at the start, and the model's last norm reads
+    their sum).  Each sublayer ``q`` (1: the mixer, 2: the feed-forward) has three small tensors, ``hc<q>.in [S]``,
+    ``hc<q>.out [S]`` and ``hc<q>.mix [S, S]`` (from-stream by to-stream):
+
+        u = sum_s in[s] X[s];  y = sublayer(norm(u));  X'[t] = sum_s mix[s, t] X[s] + out[t] y   (all t at once)
+
+    As the other arrangements leave the addition of a sublayer's output to the norm that follows, this one
+    leaves the update: a sublayer's output goes on as :class:`~fastgen_amd.kernels.ops.StreamUpdate`, and one
+    kernel (``ops.streams_step``) applies it, forms the next ``u`` and norms it, all in fp32.  A layer without a
+    feed-forward has the first half only.  Options: ``streams``, ``dim``, ``learned`` (False: there are no such
+    tensors, every weight is one: with one stream that is the plain pre-norm layer); the spec's prefix is the
+    layer's."""
+
+    folds_norms = False
+
+    def __init__(self, spec, mixer: Mixer, ffn: Optional[FeedForward], mixer_norm: Norm, ffn_norm: Optional[Norm]) -> None:
+        super().__init__(spec)
+        self.streams = int(spec.options["streams"])
+        self.learned = bool(spec.options.get("learned", True))
+        if not 1 <= self.streams <= ops.STREAMS_MAX:
+            raise ValueError(f"{self.prefix}: {self.streams} streams are not supported (1 to {ops.STREAMS_MAX})")
+        if ffn is not None and ffn_norm is None:
+            raise ValueError("a feed-forward needs its norm")
+        self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
+        _no_output_bias(ffn, "hyper-connection")
+        self.weights: dict = {}
+
+    def _sublayers(self):
+        return ("hc1", "hc2") if self.ffn is not None else ("hc1",)
+
+    def tensor_specs(self):
+        S, specs = self.streams, []
+        for q in self._sublayers() if self.learned else ():
+            specs += [TensorSpec(self._name(f"{q}.in"), (S,), VECTOR, ("one_plus_normal", 0.1)),
+                      TensorSpec(self._name(f"{q}.out"), (S,), VECTOR, ("one_plus_normal", 0.1)),
+                      TensorSpec(self._name(f"{q}.mix"), (S, S), VECTOR, ("eye_plus_normal", 0.1))]
+        return specs
+
+    def load(self, tensors, dtype, device) -> None:
+        for q in self._sublayers():
+            for n in ("in", "out", "mix"):
+                shape = (self.streams, self.streams) if n == "mix" else (self.streams,)
+                self.weights[f"{q}.{n}"] = (tensors[self._name(f"{q}.{n}")].to(device=device, dtype=torch.float32).contiguous()
+                                            if self.learned else torch.ones(shape, dtype=torch.float32, device=device))
+
+    def _read(self, h: torch.Tensor, pending, q: str, norm: Norm, dtype: torch.dtype) -> torch.Tensor:
+        if h.dim() != 3 or h.shape[0] != self.streams:
+            raise ValueError(f"{self.prefix}: the model keeps no {self.streams} residual streams (ModelLayout.streams)")
+        if pending is not None and not isinstance(pending, ops.StreamUpdate):
+            raise ValueError(f"{self.prefix}: what the layer before left is no update of the streams")
+        out = torch.empty(h.shape[1:], dtype=dtype, device=h.device)
+        return ops.streams_step(h, pending, self.weights[f"{q}.in"], norm.weight, norm.eps, out)
+
+    def forward(self, h: torch.Tensor, pending, ctx: Any, store: LayerStore):
+        x = self._read(h, pending, "hc1", self.mixer_norm, ctx.act_dtype)
+        update = ops.StreamUpdate(self.mixer.forward(x, ctx, store), self.weights["hc1.mix"], self.weights["hc1.out"])
+        if self.ffn is None:
+            return update
+        x = self._read(h, update, "hc2", self.ffn_norm, ctx.act_dtype)
+        return ops.StreamUpdate(self.ffn.forward(x), self.weights["hc2.mix"], self.weights["hc2.out"])
+
+
+register_part("arrangement", "hyper_connections", HyperConnectionBlock)

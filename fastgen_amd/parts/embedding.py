@@ -38,7 +38,7 @@ class Embedding(Part):
 class LMHead(Part):
     """fp32 logits ``x W^T``; ``W`` is the head's own matrix or, when tied,
     the embedding table (``fastgen/forward.py:507-515``).  With the option ``softcap`` the logits are
-    ``cap * tanh(logits / cap)``."""
+    ``cap * tanh(logits / cap)``; with the option ``scale`` they are multiplied by that constant."""
 
     def __init__(self, spec) -> None:
         super().__init__(spec)
@@ -46,6 +46,7 @@ class LMHead(Part):
         self.dim = int(spec.options["dim"])
         self.tied_to: Optional[str] = spec.options.get("tied_to")
         self.softcap = float(spec.options.get("softcap") or 0.0)
+        self.scale = float(spec.options.get("scale", 1.0))
         self.weight: Optional[StreamedMatrix] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -66,6 +67,8 @@ class LMHead(Part):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = linear(x, self.weight, out_dtype=torch.float32)
+        if self.scale != 1.0:
+            logits = ops.scale_logits(logits, self.scale)
         return ops.softcap(logits, self.softcap) if self.softcap > 0 else logits
 
 

@@ -3,7 +3,9 @@
 interleaved in groups of 8, so one product gives both and a tile of it holds
 both halves of a channel: for few rows ``silu(gate) * up`` is applied where the
 product is stored.  The option ``activation`` puts the tanh form of GELU
-(``"gelu_tanh"``) or ReLU (``"relu"``) in SiLU's place.  With the option ``bias``
+(``"gelu_tanh"``) or ReLU (``"relu"``) in SiLU's place, or the limited one (``"limited"`` with
+``limit`` and ``alpha``: ``g * sigmoid(alpha g) * (u + 1)`` of ``g = min(gate, limit)``,
+``u = clamp(up, -limit, limit)``).  With the option ``bias``
 every projection has a bias: the gate's and the up projection's are added in
 fp32 where the activation is applied to the product's fp32 result; the down
 projection's (``output_bias``) is left to the kernel that adds the result to the
@@ -28,11 +30,15 @@ class SwiGLU(FeedForward):
         self.dim = int(spec.options["dim"])
         self.hidden_dim = int(spec.options["hidden_dim"])
         self.activation = spec.options.get("activation", "silu")
-        if self.activation not in ("silu", "gelu_tanh", "relu"):
-            raise ValueError(f"{self.prefix}: activation {self.activation!r} is not supported ('silu', 'gelu_tanh', 'relu')")
+        if self.activation not in ("silu", "gelu_tanh", "relu", "limited"):
+            raise ValueError(f"{self.prefix}: activation {self.activation!r} is not supported ('silu', 'gelu_tanh', 'relu',"
+                             " 'limited')")
+        self.limit, self.alpha = float(spec.options.get("limit") or 0.0), float(spec.options.get("alpha", 1.0))
+        if (self.activation == "limited") != (self.limit > 0):
+            raise ValueError(f"{self.prefix}: the limited activation, and only it, needs a positive limit")
         self.bias = bool(spec.options.get("bias", False))
         # the activation in a kernel of its own, on the product's rows: what the products' epilogues do not cover
-        self.separate = self.bias or self.activation == "relu"
+        self.separate = self.bias or self.activation in ("relu", "limited")
         self.folds_norms = not self.separate
         self.b_gate_up: Optional[torch.Tensor] = None
         self.output_bias: Optional[torch.Tensor] = None
@@ -78,7 +84,7 @@ class SwiGLU(FeedForward):
         if self.separate:
             x = x.materialize() if isinstance(x, ops.ScaledRows) else x
             gate_up = linear(x, self.w_gate_up, out_dtype=torch.float32)
-            act = ops.gated_mul(gate_up, self.b_gate_up, self.activation, x.dtype)
+            act = ops.gated_mul(gate_up, self.b_gate_up, self.activation, x.dtype, None, self.limit, self.alpha)
             return linear(act, self.w_down, partials_ok=True)
         act = linear(x, self.w_gate_up, epilogue=f"{self.activation}_mul")
         return linear(act, self.w_down, partials_ok=True, residual=then)

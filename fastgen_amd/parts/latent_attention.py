@@ -1,5 +1,5 @@
-"""Attention through latents: queries come from a narrow normed latent, keys and values from
-another one that is all the cache holds.
+"""Attention through latents: queries come from a narrow normed latent (or, without ``q_rank``, from one
+projection of the mixer's input), keys and values from another one that is all the cache holds.
 
 Per token the cache keeps one row for all heads: the normed key/value latent ``c`` (``kv_rank``
 wide) followed by one rotated key part ``r`` (``rot_dim`` wide) that the heads share.  Head ``h``'s key
@@ -11,8 +11,9 @@ with one key/value head whose keys are the cached rows and whose values are thei
 (a product per head again), times a sigmoid gate per head, into the output projection.
 
 Options: ``dim``, ``n_heads``, ``head_dim`` (the plain part of a query or key), ``rot_dim``,
-``v_head_dim``, ``kv_rank``, ``q_rank``, ``scale``, ``window``, ``sink``, ``head_gate``, ``eps`` (of the
-latents' norms), ``position`` (a rotary scheme over ``rot_dim`` dimensions).
+``v_head_dim``, ``kv_rank``, ``q_rank`` (None: no query latent; the tensor ``q_proj.weight`` gives the heads' queries
+directly), ``scale``, ``window``, ``block`` (a mask of blocks of that many positions instead), ``sink``, ``head_gate``,
+``eps`` (of the latents' norms), ``position`` (a rotary scheme over ``rot_dim`` dimensions).
 """
 
 from __future__ import annotations
@@ -36,9 +37,12 @@ class LatentAttention(Mixer):
         self.rot_dim = int(o["rot_dim"])
         self.v_head_dim = int(o["v_head_dim"])
         self.kv_rank = int(o["kv_rank"])
-        self.q_rank = int(o["q_rank"])
+        self.q_rank: Optional[int] = int(o["q_rank"]) if o.get("q_rank") else None
         self.scale = float(o.get("scale", (self.head_dim + self.rot_dim) ** -0.5))
         self.window: Optional[int] = o.get("window") or None
+        self.block: Optional[int] = o.get("block") or None
+        if self.block and self.window:
+            raise ValueError(f"{self.prefix}: a mask of blocks and a sliding window do not go together")
         self.sink = bool(o.get("sink", False))
         self.head_gate = bool(o.get("head_gate", False))
         self.eps = float(o["eps"])
@@ -47,7 +51,7 @@ class LatentAttention(Mixer):
         if self.position.rotary_dim != self.rot_dim:
             raise ValueError(f"{self.prefix}: the rotary scheme turns {self.position.rotary_dim} dimensions, rot_dim is {self.rot_dim}")
         for name, v in (("head_dim", self.head_dim), ("rot_dim", self.rot_dim), ("kv_rank", self.kv_rank),
-                        ("q_rank", self.q_rank), ("v_head_dim", self.v_head_dim)):
+                        ("q_rank", self.q_rank or 2), ("v_head_dim", self.v_head_dim)):
             if v <= 0 or v % 2:
                 raise ValueError(f"{self.prefix}: {name}={v} must be positive and even")
         # a cached row: the latent, the shared rotated part, zeros up to a multiple of 16
@@ -63,9 +67,13 @@ class LatentAttention(Mixer):
     def tensor_specs(self) -> List[TensorSpec]:
         H, d, r, e, R, Q = self.n_heads, self.head_dim, self.rot_dim, self.v_head_dim, self.kv_rank, self.q_rank
         one = ("one_plus_normal", 0.01)
-        specs = [
-            TensorSpec(self._name("q_down.weight"), (Q, self.dim)), TensorSpec(self._name("q_down_norm.weight"), (Q,), VECTOR, one),
-            TensorSpec(self._name("q_up.weight"), (H * (d + r), Q)),
+        if Q is None:
+            specs = [TensorSpec(self._name("q_proj.weight"), (H * (d + r), self.dim))]
+        else:
+            specs = [TensorSpec(self._name("q_down.weight"), (Q, self.dim)),
+                     TensorSpec(self._name("q_down_norm.weight"), (Q,), VECTOR, one),
+                     TensorSpec(self._name("q_up.weight"), (H * (d + r), Q))]
+        specs += [
             TensorSpec(self._name("kv_down.weight"), (R + r, self.dim)),
             TensorSpec(self._name("kv_down_norm.weight"), (R,), VECTOR, one),
             TensorSpec(self._name("k_up.weight"), (H * d, R)), TensorSpec(self._name("v_up.weight"), (H * e, R)),
@@ -94,16 +102,20 @@ class LatentAttention(Mixer):
         f32 = lambda name: t(name).to(device=device, dtype=torch.float32).contiguous()
         # one matrix for everything that reads the mixer's input: the query latent, the key/value latent with
         # the shared rotated part, the heads' gates
-        mats = [t("q_down.weight"), self._interleave(t("kv_down.weight"), 1, R + r, R)]
+        # (without a query latent: the heads' queries themselves come first)
+        first = t("q_down.weight") if self.q_rank else self._interleave(t("q_proj.weight"), H, d + r, d)
+        mats = [first, self._interleave(t("kv_down.weight"), 1, R + r, R)]
         if self.head_gate:
             mats.append(t("gate_proj.weight"))
         self.w_in = streamed(place(torch.cat(mats, dim=0), MATRIX, dtype, device))
-        self.w_uq = streamed(place(self._interleave(t("q_up.weight"), H, d + r, d), MATRIX, dtype, device))
+        if self.q_rank:
+            self.w_uq = streamed(place(self._interleave(t("q_up.weight"), H, d + r, d), MATRIX, dtype, device))
         # per head: W_uk^T [R, d] carries a query into the latent's space, W_uv [e, R] a head's output out of it
         self.w_uk_t = place(t("k_up.weight").view(H, d, R).transpose(1, 2), MATRIX, dtype, device)
         self.w_uv = place(t("v_up.weight").view(H, e, R), MATRIX, dtype, device)
         self.wo = streamed(place(t("o_proj.weight"), MATRIX, dtype, device))
-        self.dq_norm, self.dkv_norm = f32("q_down_norm.weight"), f32("kv_down_norm.weight")
+        self.dq_norm = f32("q_down_norm.weight") if self.q_rank else None
+        self.dkv_norm = f32("kv_down_norm.weight")
         self.sinks = f32("sinks") if self.sink else None
         self.freqs = self.position.frequencies_on(device)
 
@@ -119,23 +131,34 @@ class LatentAttention(Mixer):
         table = ctx.scratch.get(key)
         if table is None:
             table = ctx.scratch[key] = ops.rope_table(ctx.positions, self.freqs)
-        rows = linear(x, self.w_in, out_dtype=torch.float32)  # [T, Q | R + r | H] fp32
-        cq = torch.empty((T, Q), dtype=x.dtype, device=x.device)
+        rows = linear(x, self.w_in, out_dtype=torch.float32)  # [T, Q (or H (d + r)) | R + r | H] fp32
         own = store.owns
-        ops.heads_prepare(
-            rows, None, self.eps, n_q=1, q_col=0, q_width=Q, q_norm=self.dq_norm, q_norm_dims=Q, q_out=cq, q_out_width=Q,
-            n_kv=1 if own else 0, k_col=Q, k_width=R + r, k_norm=self.dkv_norm, k_norm_dims=R, v_col=-1, v_width=R,
-            table=table, rot_start=R, rotary_dim=r, rotate_q=False, rotate_k=True,
-            slots=group.slots if own else None, k_pages=store.k_pages if own else None,
-            v_pages=store.v_pages if own else None)
-        q = linear(cq, self.w_uq)  # [T, H * (d + r)]
-        ops.heads_prepare(q, None, self.eps, n_q=H, q_col=0, q_width=d + r, q_out=q, q_out_width=d + r,
-                          table=table, rot_start=d, rotary_dim=r)
+        if Q is None:
+            Q = H * (d + r)  # the first columns are the heads' queries
+            if own:
+                ops.heads_prepare(
+                    rows, None, self.eps, n_kv=1, k_col=Q, k_width=R + r, k_norm=self.dkv_norm, k_norm_dims=R, v_col=-1,
+                    v_width=R, table=table, rot_start=R, rotary_dim=r, rotate_q=False, rotate_k=True, slots=group.slots,
+                    k_pages=store.k_pages, v_pages=store.v_pages)
+            q = torch.empty((T, Q), dtype=x.dtype, device=x.device)
+            ops.heads_prepare(rows, None, self.eps, n_q=H, q_col=0, q_width=d + r, q_out=q, q_out_width=d + r,
+                              table=table, rot_start=d, rotary_dim=r)
+        else:
+            cq = torch.empty((T, Q), dtype=x.dtype, device=x.device)
+            ops.heads_prepare(
+                rows, None, self.eps, n_q=1, q_col=0, q_width=Q, q_norm=self.dq_norm, q_norm_dims=Q, q_out=cq, q_out_width=Q,
+                n_kv=1 if own else 0, k_col=Q, k_width=R + r, k_norm=self.dkv_norm, k_norm_dims=R, v_col=-1, v_width=R,
+                table=table, rot_start=R, rotary_dim=r, rotate_q=False, rotate_k=True,
+                slots=group.slots if own else None, k_pages=store.k_pages if own else None,
+                v_pages=store.v_pages if own else None)
+            q = linear(cq, self.w_uq)  # [T, H * (d + r)]
+            ops.heads_prepare(q, None, self.eps, n_q=H, q_col=0, q_width=d + r, q_out=q, q_out_width=d + r,
+                              table=table, rot_start=d, rotary_dim=r)
         q_lat = torch.empty((T, H * hc), dtype=x.dtype, device=x.device)
         ops.head_linear(q, d + r, self.w_uk_t, q_lat, hc, tail=r)
         lat = torch.empty_like(q_lat)
-        ops.paged_attention(q_lat, lat, store.k_pages, store.v_pages, group, ctx, H, self.scale, self.window or 0,
-                            exact_weights=self.exact_weights, sinks=self.sinks)
+        ops.paged_attention(q_lat, lat, store.k_pages, store.v_pages, group, ctx, H, self.scale,
+                            ops.block_mask(self.block) if self.block else (self.window or 0), exact_weights=self.exact_weights, sinks=self.sinks)
         out = torch.empty((T, H * e), dtype=x.dtype, device=x.device)
         ops.head_linear(lat, hc, self.w_uv, out, e, gate=rows[:, Q + R + r:] if self.head_gate else None)
         return linear(out, self.wo, partials_ok=True)

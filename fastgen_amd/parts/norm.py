@@ -38,9 +38,12 @@ class RMSNorm(Norm):
     def forward(self, h, delta, dtype, rows=None):
         """``delta`` may be :class:`~fastgen_amd.kernels.ops.PostNormed`: a sublayer's output that is normed
         itself before it is added (the norm behind a sublayer); one kernel does that norm, the addition and
-        this norm."""
-        n = h.shape[0] if rows is None else rows.numel()
+        this norm.  ``h`` may be several residual streams ``[S, T, dim]`` (``delta``: the
+        :class:`~fastgen_amd.kernels.ops.StreamUpdate` still to be applied, or None): their sum is normed."""
+        n = h.shape[-2] if rows is None else rows.numel()
         out = torch.empty((n, self.dim), dtype=dtype, device=h.device)
+        if h.dim() == 3:
+            return ops.streams_step(h, delta, None, self.weight, self.eps, out, rows)
         if isinstance(delta, ops.PostNormed):
             return ops.post_add_rmsnorm(h, delta.rows, delta.weight, delta.eps, self.weight, self.eps, out, rows,
                                         delta_bias=delta.bias)

@@ -123,6 +123,8 @@ class RandomSource(TensorSource):
         t.normal_(0.0, std, generator=g)
         if kind == "one_plus_normal":
             t += 1.0
+        elif kind == "eye_plus_normal":  # a square matrix around the identity
+            t += torch.eye(spec.shape[0], spec.shape[1], dtype=torch.float32, device=self.device)
         elif kind != "normal":
             raise ValueError(f"unknown init {kind!r} for {name}")
         return t.to(self.dtype)

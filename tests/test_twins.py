@@ -26,7 +26,7 @@ KERNEL_OPS = ["embed", "add_rmsnorm", "rmsnorm", "silu_mul", "rope_table", "rope
               "gemm_skinny_qkv", "gemm_tiled", "sample", "logprob", "stream_add", "add_rows", "gate_mul", "moe_route",
               "moe_sort", "moe_gate_up", "moe_down", "moe_combine", "gelu_mul", "post_add_rmsnorm", "softcap",
               "heads_prepare", "head_linear", "head_norm_gate", "decay_scan", "gated_mul", "causal_conv", "selective_scan",
-              "sigmoid_attention"]
+              "sigmoid_attention", "scale_logits", "head_diff_norm", "streams_spread", "streams_step"]
 
 
 @pytest.mark.parametrize("name", KERNEL_OPS + ["interleave_gate_up"])
