@@ -226,3 +226,124 @@ def plain_forward(weights: Mapping[str, torch.Tensor], config: Mapping, tokens: 
             layers_out.append(X.sum(0))
     x = plain_rms(X.sum(0), w["final.norm"], eps).to(dtype)
     return (_hi(x) @ _hi(w["embed"]).T) * config.get("logit_scale", 1.0)
+
+
+def plain_greedy(weights: Mapping[str, torch.Tensor], config: Mapping, prompt: List[int], n_new: int,
+                 dtype: torch.dtype = torch.float32) -> List[int]:
+    """``n_new`` tokens, each the argmax of the last position's logits of the whole sequence so far."""
+    seq, out = list(prompt), []
+    for _ in range(n_new):
+        tok = int(plain_forward(weights, config, seq, dtype)[-1].argmax())
+        out.append(tok)
+        seq.append(tok)
+    return out
+
+
+# --------------------------------------------------------------------- weights
+def plain_weights(config: Mapping, seed: int, stored: torch.dtype = torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Random tensors of a configuration, by the names of the checkpoint, with the values that ``stored`` can hold
+    (as float32)."""
+    g = torch.Generator().manual_seed(seed)
+    D, V, S = config["width"], config["vocab"], int(config.get("streams", 1))
+    w: Dict[str, torch.Tensor] = {}
+
+    def mat(name, rows, cols, std=None):
+        w[name] = torch.randn(rows, cols, generator=g) * (std if std is not None else cols ** -0.5)
+
+    def vec(name, n, mean=0.0, std=0.1):
+        w[name] = mean + std * torch.randn(n, generator=g)
+
+    mat("embed", V, D, 1.0)
+    vec("final.norm", D, 1.0)
+    for i, layer in enumerate(config["layers"]):
+        m, p = layer["mixer"], f"l{i}"
+        vec(f"{p}.norm1", D, 1.0)
+        subs = ["hc1"]
+        if layer["type"] == "attention":
+            H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            mat(f"{p}.mix.q", H * 2 * d, D)
+            if m.get("kv_from") is None:
+                mat(f"{p}.mix.k", G * 2 * d, D)
+                mat(f"{p}.mix.v", G * e, D)
+            for n in ("lq1", "lk1", "lq2", "lk2"):
+                vec(f"{p}.mix.{n}", d, 0.0, 0.3)
+            mat(f"{p}.mix.o", D, H * e)
+        else:
+            H, d, r, e, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+            mat(f"{p}.mix.q", H * (d + r), D)
+            mat(f"{p}.mix.dkv", R + r, D)
+            vec(f"{p}.mix.dkv.norm", R, 1.0)
+            mat(f"{p}.mix.uk", H * d, R)
+            mat(f"{p}.mix.uv", H * e, R)
+            vec(f"{p}.mix.sink", H, 0.0, 1.0)
+            mat(f"{p}.mix.o", D, H * e)
+        mlp = layer.get("mlp")
+        if mlp is not None:
+            subs.append("hc2")
+            vec(f"{p}.norm2", D, 1.0)
+            E, ff = mlp["router"]["experts"], mlp["expert"]["ff"]
+            mat(f"{p}.mlp.router", E, D, 0.5 * D ** -0.5 * 3)
+            vec(f"{p}.mlp.correction", E, 0.0, 0.05)
+            for e_ in range(E):
+                mat(f"{p}.mlp.e{e_}.gate", ff, D, 2 * D ** -0.5)
+                mat(f"{p}.mlp.e{e_}.up", ff, D, 2 * D ** -0.5)
+                mat(f"{p}.mlp.e{e_}.down", D, ff)
+            if mlp.get("shared"):
+                sf = mlp["shared"]["ff"]
+                mat(f"{p}.mlp.shared.gate", sf, D, 2 * D ** -0.5)
+                mat(f"{p}.mlp.shared.up", sf, D, 2 * D ** -0.5)
+                mat(f"{p}.mlp.shared.down", D, sf)
+                mat(f"{p}.mlp.shared.sg", 1, D)
+        for q in subs:
+            vec(f"{p}.{q}.in", S, 1.0 / S, 0.2)
+            vec(f"{p}.{q}.out", S, 1.0, 0.3)
+            w[f"{p}.{q}.mix"] = torch.eye(S) + 0.2 * torch.randn(S, S, generator=g)
+    return {k: v.to(stored).float() for k, v in w.items()}
+
+
+# ---------------------------------------------------------------- configurations
+def _moe(experts, top, ff, limit, shared=None):
+    out = {"kind": "moe", "expert": {"ff": ff, "limit": limit}, "router": {"experts": experts, "top": top}}
+    if shared is not None:
+        out["shared"] = {"ff": shared[0], "limit": shared[1]}
+    return out
+
+
+def _diff(heads, kv, dim, vdim, rot, block, diff, base=5000.0, kv_from=None):
+    m = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "diff": diff,
+         "rot": {"base": base, "dims": rot}}
+    if block:
+        m["mask"] = {"size": block}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return m
+
+
+def _latent(heads, dim, rot, vdim, rank, base=300.0):
+    return {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "scale": (dim + rot) ** -0.5,
+            "rot": {"base": base, "dims": rot}}
+
+
+# both mixers, a layer on another's keys with a block size of its own, a layer without feed-forward, two streams
+PAIR = {"architecture": "Sodotar", "width": 64, "vocab": 96, "norm": {"eps": 1e-5}, "streams": 2, "logit_scale": 0.5,
+        "layers": [
+            {"type": "attention", "mixer": _diff(4, 2, 16, 32, 8, 24, 0.3), "mlp": _moe(6, 2, 24, 1.0, (40, 1.5))},
+            {"type": "latent_attention", "mixer": _latent(3, 16, 8, 24, 24), "mlp": _moe(5, 2, 32, 2.0, (16, 1.0))},
+            {"type": "attention", "mixer": _diff(4, 2, 16, 32, 8, 40, 0.5, kv_from=0), "mlp": None},
+            {"type": "latent_attention", "mixer": _latent(2, 8, 16, 40, 40), "mlp": _moe(6, 2, 24, 1.0, (40, 1.5))}]}
+# one stream, heads that are no power of two, one head a group, values narrower than keys, every dimension rotated,
+# no mask, every expert chosen, widths that are no multiple of 8, no shared expert, logits as they are
+ODD = {"architecture": "Sodotar", "width": 72, "vocab": 50, "norm": {"eps": 1e-6}, "streams": 1,
+       "layers": [
+           {"type": "attention", "mixer": _diff(3, 3, 24, 16, 24, None, 0.8), "mlp": _moe(3, 3, 20, 0.7)},
+           {"type": "latent_attention", "mixer": _latent(1, 24, 4, 10, 18), "mlp": _moe(4, 1, 12, 1.2, (20, 0.9))},
+           {"type": "attention", "mixer": _diff(6, 2, 8, 8, 2, 7, 0.2), "mlp": _moe(4, 1, 12, 1.2, (20, 0.9))}]}
+# four streams; twenty heads on one key head (more than the matrix-core kernels group); blocks of one page's size
+WIDE = {"architecture": "Sodotar", "width": 64, "vocab": 80, "norm": {"eps": 1e-5}, "streams": 4, "logit_scale": 1.5,
+        "layers": [
+            {"type": "attention", "mixer": _diff(20, 1, 8, 16, 4, 16, 0.4), "mlp": _moe(8, 3, 16, 1.5, (24, 2.0))},
+            {"type": "attention", "mixer": _diff(20, 1, 8, 16, 4, 64, 0.6, kv_from=0), "mlp": _moe(8, 3, 16, 1.5, (24, 2.0))}]}
+ONLY_DIFF = {"architecture": "Sodotar", "width": 48, "vocab": 64, "norm": {"eps": 1e-5}, "streams": 1, "logit_scale": 1.0,
+             "layers": [{"type": "attention", "mixer": _diff(2, 1, 16, 16, 8, 32, 0.5), "mlp": None}]}
+ONLY_LATENT = {"architecture": "Sodotar", "width": 48, "vocab": 64, "norm": {"eps": 1e-5}, "streams": 1, "logit_scale": 1.0,
+               "layers": [{"type": "latent_attention", "mixer": _latent(2, 16, 8, 16, 32), "mlp": None}]}
