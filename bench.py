@@ -8,6 +8,7 @@
     python bench.py --workload buderax      # the Buderax design beside the dense Llama at equal sizes
     python bench.py --workload gisodra      # the Gisodra design beside the dense Llama at equal sizes
     python bench.py --workload zudisun      # the Zudisun design beside Gisodra and the dense Llama at equal sizes
+    python bench.py --workload sodotar      # the Sodotar design beside Gisodra and the dense Llama at equal sizes
 
 The model has the layer sizes of Llama 3.1 8B (32 layers, hidden 4096, 32
 heads, 8 kv heads, head size 128, feed-forward 14336, vocabulary 128256,
@@ -672,6 +673,195 @@ def zudisun_workload(prefill_tokens: int = 2048, batch: int = 8, context: int = 
     return 0
 
 
+# Sodotar at sizes that resemble a real model's layers: eight layers in the order differential attention, latent
+# attention, differential attention on the first one's keys, latent attention, twice, each with a routed
+# feed-forward and a gated shared expert, four residual streams.  A differential layer has half the heads of the
+# models beside it, two maps a head and values twice as wide (as many score maps and as many value columns).
+# Beside it: Gisodra (the framework's closest model: attention layers that read another layer's cache, latent
+# attention) and the dense Llama, both of the same width, heads, head size and number of layers, whose dense
+# feed-forward is as wide as the experts a token uses plus the shared one.
+SODOTAR_SIZES = {
+    "w1024": dict(width=1024, heads=16, kv_heads=4, dim=64, block=1024, lat_dim=64, rot_dim=32, kv_rank=192, streams=4,
+                  experts=16, top=2, expert_ff=704, shared_ff=1408, vocab=32000),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, block=4096, lat_dim=128, rot_dim=64, kv_rank=192, streams=4,
+                  experts=32, top=4, expert_ff=768, shared_ff=2560, vocab=32000),
+}
+
+
+def _sodotar_configs(z: dict):
+    mlp = dict(kind="moe", router=dict(experts=z["experts"], top=z["top"]), expert=dict(ff=z["expert_ff"], limit=7.0),
+               shared=dict(ff=z["shared_ff"], limit=7.0))
+    diff = lambda **more: dict(type="attention", mlp=mlp, mixer=dict(
+        heads=z["heads"] // 2, kv_heads=z["kv_heads"] // 2, dim=z["dim"], vdim=2 * z["dim"], scale=z["dim"] ** -0.5, diff=0.8,
+        mask=dict(size=z["block"]), rot=dict(base=500000.0, dims=z["dim"]), **more))
+    latent = dict(type="latent_attention", mlp=mlp, mixer=dict(
+        heads=z["heads"], dim=z["lat_dim"], rot_dim=z["rot_dim"], vdim=z["dim"], kv_rank=z["kv_rank"],
+        scale=(z["lat_dim"] + z["rot_dim"]) ** -0.5, rot=dict(base=1000000.0, dims=z["rot_dim"])))
+    layers = [diff(), latent, diff(kv_from=0), latent, diff(), latent, diff(kv_from=4), latent]
+    new = dict(architecture="Sodotar", width=z["width"], vocab=z["vocab"], norm=dict(eps=1e-6), streams=z["streams"],
+               logit_scale=0.5, layers=layers)
+    ff = z["top"] * z["expert_ff"] + z["shared_ff"]
+    g = dict(GISODRA_SIZES["w1024" if z["width"] == 1024 else "w2048"], ff=ff)
+    hybrid, _ = _gisodra_configs(g)
+    dense = dict(architectures=["LlamaForCausalLM"], hidden_size=z["width"], intermediate_size=ff,
+                 num_hidden_layers=len(layers), num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"],
+                 rms_norm_eps=1e-6, vocab_size=z["vocab"], rope_theta=500000.0, rope_scaling=None,
+                 tie_word_embeddings=True, max_position_embeddings=131072)
+    return new, hybrid, dense
+
+
+def _sodotar_kernels(z: dict, rows: int, context: int) -> dict:
+    """The design's own kernels at ``rows`` tokens (one prompt of ``rows`` tokens, or ``rows`` sequences of one
+    token at ``context`` cached ones), each beside the like kernel of the closest model on operands of the same
+    size: microseconds, and the shares of the memory roofline (the bytes the kernel has to move) and of the
+    matrix cores' (its products' flops)."""
+    import numpy as np
+    import torch
+
+    from fastgen_amd.kernels import ops
+
+    D, H, G, d, P, S = z["width"], z["heads"], z["kv_heads"], z["dim"], PAGE, z["streams"]
+    Hd, Gd, e = H // 2, G // 2, 2 * d  # the differential layer: heads, key/value heads, value width
+    g = torch.Generator(device="cuda").manual_seed(rows)
+    rnd = lambda *shape: (torch.randn(*shape, generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+    f32 = lambda *shape: torch.randn(*shape, generator=g, device="cuda")
+    decode = rows <= 16
+    out = {}
+
+    def put(name, fn, nbytes, flops=0):
+        t = _time(fn)
+        out[name] = {"us": round(t * 1e6, 1), "hbm_frac": round(nbytes / t / PEAK_HBM, 4),
+                     "mfma_frac": round(flops / t / PEAK_FLOPS["bf16"], 4)}
+
+    # the streams' update, sum and norm; beside the one stream's addition and norm
+    x, delta, w = f32(S, rows, D), rnd(rows, D), rnd(D)
+    upd = ops.StreamUpdate(delta, f32(S, S), f32(S))
+    normed = torch.empty(rows, D, dtype=torch.bfloat16, device="cuda")
+    put("streams_step", lambda: ops.streams_step(x, upd, f32(S), w, 1e-6, normed), rows * D * (8 * S + 2 + 2))
+    h = f32(rows, D)
+    put("add_rmsnorm (one stream)", lambda: ops.add_rmsnorm(h, delta, w, 1e-6, normed), rows * D * (4 + 4 + 2 + 2))
+    # between the q/k/v product and the attention: rotation, padding, cache write (the value goes in with both maps)
+    n_seqs = rows if decode else 1
+    keys = context + 1 if decode else rows
+    pages_seq = -(-keys // P)
+    n_pages = n_seqs * pages_seq
+    hc = -(-max(d, e) // 16) * 16
+    width = 2 * Hd * d + 2 * Gd * d + 2 * Gd * e
+    src = f32(rows, width)
+    kp, vp = rnd(n_pages, 2 * Gd, P, hc), rnd(n_pages, 2 * Gd, hc, P)
+    table = ops.rope_table(torch.arange(rows, dtype=torch.int32, device="cuda"), f32(d // 2).abs())
+    bt = torch.arange(n_pages, dtype=torch.int32, device="cuda").view(n_seqs, pages_seq)
+    if decode:
+        slots = (torch.arange(rows, dtype=torch.int32, device="cuda") * pages_seq * P + context).contiguous()
+    else:
+        slots = torch.arange(rows, dtype=torch.int32, device="cuda")
+    q = torch.empty(rows, 2 * Hd * hc, dtype=torch.bfloat16, device="cuda")
+    put("heads_prepare (two maps a head)", lambda: ops.heads_prepare(
+        src, None, 1e-6, n_q=2 * Hd, q_col=0, q_width=d, q_out=q, q_out_width=hc, n_kv=2 * Gd, k_col=2 * Hd * d, k_width=d,
+        v_col=2 * Hd * d + 2 * Gd * d, v_width=e, table=table, rot_start=0, rotary_dim=d, slots=slots, k_pages=kp, v_pages=vp),
+        src.numel() * 4 + rows * (2 * Hd * hc + 4 * Gd * hc) * 2)
+    src_g, nw = f32(rows, (H + 2 * G) * d), f32(d)
+    kg, vg = rnd(n_pages, G, P, d), rnd(n_pages, G, d, P)
+    qg = torch.empty(rows, H * d, dtype=torch.bfloat16, device="cuda")
+    put("heads_prepare (gisodra attention)", lambda: ops.heads_prepare(
+        src_g, None, 1e-6, n_q=H, q_col=0, q_width=d, q_norm=nw, q_norm_dims=d, q_out=qg, q_out_width=d, n_kv=G, k_col=H * d,
+        k_width=d, k_norm=nw, k_norm_dims=d, v_col=(H + G) * d, v_width=d, slots=slots, k_pages=kg, v_pages=vg),
+        src_g.numel() * 4 + rows * (H + 2 * G) * d * 2)
+    # the attention itself: 2 Hd maps over 2 Gd key heads of the padded width and a mask of blocks, beside H heads
+    # over G key heads of width d; the bytes are the keys and values that have to be read (a value once)
+    if decode:
+        q_lens, q_start, n_cached = [1] * rows, list(range(rows + 1)), [context] * rows
+    else:
+        q_lens, q_start, n_cached = [rows], [0, rows], [0]
+    def attention(name, qq, k_pages, v_pages, heads, kv, window, need_bytes, flops):
+        width = k_pages.shape[3]
+        small, big = ops.attention_items(np.array(q_lens), np.array(q_start), np.array(n_cached), heads // kv,
+                                         ops.attention_tile_rows(width, False, True))
+        both = ops.upload(np.concatenate([small, big]).reshape(-1), torch.int32, "cuda")
+        sm, bg = (both[: small.size] if small.size else None), (both[small.size:] if big.size else None)
+        o = torch.empty(rows, heads * width, dtype=torch.bfloat16, device="cuda")
+        put(name, lambda: ops.paged_attention_mfma(qq, o, k_pages, v_pages, bt, sm, bg, heads, 0.1, window, exact_weights=True),
+            need_bytes, flops)
+    seen = n_seqs * keys if decode else rows  # keys a sequence's tokens read (a prompt: each page once a tile row)
+    pairs = n_seqs * keys if decode else rows * (rows + 1) // 2
+    attention("attention (two maps a head, blocks)", q, kp, vp, 2 * Hd, 2 * Gd, ops.block_mask(z["block"]),
+              seen * (2 * Gd * d + Gd * e) * 2, 2 * pairs * 2 * Hd * (d + e))
+    attention("attention (gisodra: H heads)", qg, kg, vg, H, G, 0, seen * 2 * G * d * 2, 2 * pairs * H * 2 * d)
+    att = rnd(rows, 2 * Hd * hc)
+    o = torch.empty(rows, Hd * e, dtype=torch.bfloat16, device="cuda")
+    put("head_diff_norm", lambda: ops.head_diff_norm(att, hc, o, Hd, Hd // Gd, e, 0.6, 1e-6, 0.2), rows * (2 * Hd * e + Hd * e) * 2)
+    x32, gate16, nwe = f32(rows, H * d), rnd(rows, H * d), f32(d)
+    og = torch.empty(rows, H * d, dtype=torch.bfloat16, device="cuda")
+    put("head_norm_gate (gisodra)", lambda: ops.head_norm_gate(x32, nwe, 1e-6, gate16, H, og), rows * H * d * (4 + 2 + 2))
+    # the router: softmax over all experts, correction, the shared expert's gate row; beside softmax over the chosen
+    E, top, F = z["experts"], z["top"], z["expert_ff"]
+    xr, router, corr = rnd(rows, D), f32(E + 1, D) * 0.05, f32(E) * 0.01
+    put("moe_route (softmax over all, gate row)", lambda: ops.moe_route(xr, router, None, top, False, corr, 1, 1, 1.0, True, 1),
+        router.numel() * 4 + rows * D * 2)
+    r2 = router[:E].contiguous()
+    put("moe_route (buderax)", lambda: ops.moe_route(xr, r2, None, top), r2.numel() * 4 + rows * D * 2)
+    # the experts' first product with the limited activation, beside the same with SiLU
+    choice, _ = ops.moe_route(xr, r2, None, top)
+    tile_rows = 16 if decode else (128 if rows * top / E >= 96 else 64)
+    sorted_, tiles = ops.moe_sort(choice, E, tile_rows)
+    wg, wu = rnd(E, F, D), rnd(E, F, D)
+    used = min(E, rows * top)
+    put("moe_gate_up (limited)", lambda: ops.moe_gate_up(xr, wg, wu, sorted_, tiles, top, tile_rows, 7.0, 1.702),
+        used * 2 * F * D * 2, 2 * rows * top * 2 * F * D)
+    put("moe_gate_up (silu)", lambda: ops.moe_gate_up(xr, wg, wu, sorted_, tiles, top, tile_rows), used * 2 * F * D * 2,
+        2 * rows * top * 2 * F * D)
+    # the shared expert's activation on the product's fp32 rows, and the combine with its gate
+    gu = f32(rows, 2 * z["shared_ff"])
+    put("gated_mul (limited)", lambda: ops.gated_mul(gu, None, "limited", torch.bfloat16, None, 7.0, 1.702), rows * z["shared_ff"] * (8 + 2))
+    gu16 = rnd(rows, 2 * z["shared_ff"])
+    put("silu_mul (llama)", lambda: ops.silu_mul(gu16), rows * z["shared_ff"] * (4 + 2))
+    y, wt, plus, pg = f32(rows * top, D), f32(rows, top), rnd(rows, D), f32(rows)
+    put("moe_combine (gated shared expert)", lambda: ops.moe_combine(y, wt, plus, pg), rows * D * (4 * top + 2 + 4))
+    put("moe_combine (buderax)", lambda: ops.moe_combine(y, wt, plus), rows * D * (4 * top + 2 + 4))
+    return out
+
+
+def sodotar_workload(prefill_tokens: int = 2048, batch: int = 8, context: int = 1024, steps: int = 32, warmup: int = 8) -> int:
+    """Prefill and decode throughput of Sodotar models with random bfloat16 weights beside Gisodra and dense Llama
+    models of equal sizes, and the design's own kernels beside the other models' like ones.  One JSON line."""
+    import torch
+
+    from fastgen_amd.engine import Engine
+
+    results = {}
+    for name, z in SODOTAR_SIZES.items():
+        new, hybrid, dense = _sodotar_configs(z)
+        row = {"layers": len(new["layers"])}
+        for label, cfg in (("sodotar", new), ("gisodra", hybrid), ("llama", dense)):
+            engine = Engine.from_config(cfg, seed=5, dtype=torch.bfloat16, page_size=PAGE,
+                                        max_tokens=max(batch * (context + 256), prefill_tokens + PAGE), max_batch=batch,
+                                        max_step_tokens=prefill_tokens)
+            g = torch.Generator().manual_seed(0)
+            prompt = lambda n: torch.randint(0, z["vocab"], (n,), generator=g).tolist()
+            pre = min(engine.time_prefill(prompt(prefill_tokens), repeats=5))
+            dt = engine.time_decode([prompt(context) for _ in range(batch)], steps=steps, warmup=warmup)
+            row[label] = {"prefill_tok_s": round(prefill_tokens / pre, 1), "prefill_ms": round(pre * 1e3, 3),
+                          "decode_tok_s": round(batch * steps / dt, 1), "decode_ms_per_step": round(dt / steps * 1e3, 4),
+                          "weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
+            print(f"[bench] {name} {label}: {row[label]}", file=sys.stderr, flush=True)
+            del engine
+            torch.cuda.empty_cache()
+        row["kernels_prefill"] = _sodotar_kernels(z, prefill_tokens, context)
+        row["kernels_decode"] = _sodotar_kernels(z, batch, context)
+        print(f"[bench] {name} kernels: {row['kernels_prefill']} {row['kernels_decode']}", file=sys.stderr, flush=True)
+        results[name] = row
+    first = results[next(iter(results))]
+    print(json.dumps({
+        "metric": "Sodotar beside Gisodra and the dense Llama at equal sizes: prefill and decode tok/s", "unit": "tokens/s",
+        "value": first["sodotar"]["decode_tok_s"], "n_gpus": 1, "steps": steps, "warmup": warmup, "higher_is_better": True,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"prefill_tokens": prefill_tokens, "decode_batch": batch, "decode_context": context, "page_size": PAGE,
+                   "sizes": SODOTAR_SIZES},
+        "results": results,
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -689,9 +879,9 @@ def main() -> int:
                          " 2,048); more are fed untimed, in portions")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
-    ap.add_argument("--workload", choices=["decode", "serve", "readme", "buderax", "gisodra", "zudisun"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "serve", "readme", "buderax", "gisodra", "zudisun", "sodotar"], default="decode",
                     help="decode (default): the step benchmark; serve: continuous batching of 256 requests; "
-                         "readme: the load of the reference's README; buderax, gisodra, zudisun: that design beside the "
+                         "readme: the load of the reference's README; buderax, gisodra, zudisun, sodotar: that design beside the "
                          "dense Llama at equal sizes")
     ap.add_argument("--step-budget", type=int, default=2048, help="tokens a step of the serve workload")
     ap.add_argument("--show-choices", action="store_true",
@@ -706,6 +896,8 @@ def main() -> int:
         return readme_workload(a.shape or "8b")
     if a.workload == "gisodra":
         return gisodra_workload(prefill_tokens=a.prefill_tokens, batch=a.batch, steps=min(a.steps, 32), warmup=a.warmup)
+    if a.workload == "sodotar":
+        return sodotar_workload(prefill_tokens=a.prefill_tokens, batch=a.batch, steps=min(a.steps, 32), warmup=a.warmup)
     if a.workload == "zudisun":
         return zudisun_workload(prefill_tokens=a.prefill_tokens, batch=a.batch, steps=min(a.steps, 32), warmup=a.warmup)
     if a.workload == "buderax":
