@@ -104,6 +104,118 @@ __global__ __launch_bounds__(ST_THREADS) void streams_step_kernel(const StreamAr
   }
 }
 
+// The same with a thread holding NV runs of four consecutive elements, for dim % 4 == 0, dim <= 1024 NV and at most
+// SM streams: every load of the row (the streams, the update's rows, the norm's weight) is issued before anything
+// is computed or stored (the streams are read and written through one pointer, so the compiler would otherwise
+// keep a store of one run ahead of the next run's loads: a chain of memory round trips); the small weights are
+// read at uniform addresses.  Loads are never conditional: a thread whose run lies beyond the row reads the
+// row's last four elements and stores nothing.
+template <class T> __device__ __forceinline__ float4 load4(const T* p);
+template <> __device__ __forceinline__ float4 load4<float>(const float* p) { return *(const float4*)p; }
+template <> __device__ __forceinline__ float4 load4<bf16_t>(const bf16_t* p) {
+  const uint2 raw = *(const uint2*)p;
+  return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                     __uint_as_float(raw.y & 0xffff0000u));
+}
+template <class T> __device__ __forceinline__ void store4(T* p, float4 v);
+template <> __device__ __forceinline__ void store4<float>(float* p, float4 v) { *(float4*)p = v; }
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
+  typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+  bf16x4_t o;
+  o[0] = (__bf16)v.x; o[1] = (__bf16)v.y; o[2] = (__bf16)v.z; o[3] = (__bf16)v.w;
+  *(bf16x4_t*)p = o;
+}
+__device__ __forceinline__ float4 fma4(float w, float4 x, float4 acc) {
+  return make_float4(fmaf(w, x.x, acc.x), fmaf(w, x.y, acc.y), fmaf(w, x.z, acc.z), fmaf(w, x.w, acc.w));
+}
+
+template <class TA, class TW, int NV, int SM>
+__global__ __launch_bounds__(ST_THREADS) void streams_step_vec_kernel(const StreamArgs a) {
+  __shared__ float red[16];
+  const int S = a.n_streams, dim = a.dim;
+  const size_t tok = a.rows ? (size_t)a.rows[blockIdx.x] : (size_t)blockIdx.x;
+  const size_t stream_stride = (size_t)a.n_tokens * dim;
+  const bool pending = a.mix != nullptr;
+  int e[NV], ec[NV];
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    e[v] = (threadIdx.x + v * ST_THREADS) * 4;
+    ec[v] = min(e[v], dim - 4);
+  }
+  // the small weights first, at uniform addresses (held in scalar registers); what lies beyond S is never used
+  float mixr[SM][SM], outr[SM], inr[SM];
+#pragma unroll
+  for (int s = 0; s < SM; ++s) {
+    outr[s] = pending && s < S ? a.out_w[s] : 0.f;
+    inr[s] = a.in_w && s < S ? a.in_w[s] : 1.f;
+#pragma unroll
+    for (int t = 0; t < SM; ++t) mixr[s][t] = pending && s < S && t < S ? a.mix[s * S + t] : 0.f;
+  }
+  float4 xs[NV][SM], y[NV], w[NV];
+#pragma unroll
+  for (int v = 0; v < NV; ++v)
+#pragma unroll
+    for (int s = 0; s < SM; ++s) xs[v][s] = load4<float>(a.x + min(s, S - 1) * stream_stride + tok * dim + ec[v]);
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    y[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (a.delta) y[v] = load4<TA>((const TA*)a.delta + tok * dim + ec[v]);
+    if (a.norm_w) w[v] = load4<TW>((const TW*)a.norm_w + ec[v]);
+  }
+  if (a.parts) {
+    for (int p = 0; p < a.n_parts; ++p) {
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        const float4 d = load4<float>(a.parts + p * a.part_stride + tok * dim + ec[v]);
+        y[v] = p == 0 ? d : make_float4(y[v].x + d.x, y[v].y + d.y, y[v].z + d.z, y[v].w + d.w);
+      }
+    }
+  }
+  float4 u[NV];
+  float ss = 0.f;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (pending) {
+#pragma unroll
+      for (int t = 0; t < SM; ++t) {
+        if (t < S) {
+          float4 nv = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+          for (int s = 0; s < SM; ++s)
+            if (s < S) nv = fma4(mixr[s][t], xs[v][s], nv);
+          nv = fma4(outr[t], y[v], nv);
+          if (!a.rows && e[v] < dim) store4<float>(a.x + t * stream_stride + tok * dim + e[v], nv);
+          acc = fma4(inr[t], nv, acc);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < SM; ++s)
+        if (s < S) acc = fma4(inr[s], xs[v][s], acc);
+    }
+    u[v] = acc;
+    if (e[v] < dim) ss += acc.x * acc.x + acc.y * acc.y + acc.z * acc.z + acc.w * acc.w;
+  }
+  float rstd = 1.f;
+  if (a.norm_w) {
+    ss = block_sum(ss, red);
+    rstd = rsqrtf(ss / (float)dim + a.eps);
+  }
+  const size_t orow = (size_t)blockIdx.x * dim;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    if (e[v] >= dim) continue;
+    if (a.u_out) store4<float>(a.u_out + orow + e[v], u[v]);
+    if (a.out) {
+      const float4 n = a.norm_w ? make_float4(u[v].x * rstd * w[v].x, u[v].y * rstd * w[v].y, u[v].z * rstd * w[v].z,
+                                              u[v].w * rstd * w[v].w)
+                                : u[v];
+      store4<TA>((TA*)a.out + orow + e[v], n);
+    }
+  }
+}
+
 // n_rows: the rows of out / u_out: the tokens named by `rows`, or all n_tokens.
 extern "C" int fg_streams_step_rows(const StreamArgs* args, int n_rows, int act_dtype, int w_dtype, hipStream_t stream) {
   const StreamArgs a = *args;
@@ -114,9 +226,16 @@ extern "C" int fg_streams_step_rows(const StreamArgs* args, int n_rows, int act_
   if (!a.mix && (a.delta || a.parts)) return FG_ERR_ARG;
   if (!a.out && !a.u_out && !a.mix) return FG_ERR_ARG;
   if (!a.rows && n_rows != a.n_tokens) return FG_ERR_ARG;
+  const int S = a.n_streams;
+#define VEC(TA, TW, NV, SM) streams_step_vec_kernel<TA, TW, NV, SM><<<n_rows, ST_THREADS, 0, stream>>>(a)
 #define GO(TA, TW)                                                                               \
   do {                                                                                           \
-    if (a.dim <= 2 * ST_THREADS) streams_step_kernel<TA, TW, 2><<<n_rows, ST_THREADS, 0, stream>>>(a);       \
+    if (a.dim % 4 == 0 && a.dim <= 1024 && S <= 4) VEC(TA, TW, 1, 4);                            \
+    else if (a.dim % 4 == 0 && a.dim <= 1024) VEC(TA, TW, 1, 8);                                 \
+    else if (a.dim % 4 == 0 && a.dim <= 2048 && S <= 4) VEC(TA, TW, 2, 4);                       \
+    else if (a.dim % 4 == 0 && a.dim <= 2048) VEC(TA, TW, 2, 8);                                 \
+    else if (a.dim % 4 == 0 && a.dim <= 4096 && S <= 4) VEC(TA, TW, 4, 4);                       \
+    else if (a.dim <= 2 * ST_THREADS) streams_step_kernel<TA, TW, 2><<<n_rows, ST_THREADS, 0, stream>>>(a);  \
     else if (a.dim <= 8 * ST_THREADS) streams_step_kernel<TA, TW, 8><<<n_rows, ST_THREADS, 0, stream>>>(a);  \
     else streams_step_kernel<TA, TW, ST_MAX_PER_THREAD><<<n_rows, ST_THREADS, 0, stream>>>(a);   \
   } while (0)
@@ -126,6 +245,7 @@ extern "C" int fg_streams_step_rows(const StreamArgs* args, int n_rows, int act_
   else if (act_dtype == FG_F32 && w_dtype == FG_BF16) GO(float, bf16_t);
   else return FG_ERR_ARG;
 #undef GO
+#undef VEC
   return fg_launch_status();
 }
 
