@@ -737,7 +737,8 @@ def _sodotar_kernels(z: dict, rows: int, context: int) -> dict:
     x, delta, w = f32(S, rows, D), rnd(rows, D), rnd(D)
     upd = ops.StreamUpdate(delta, f32(S, S), f32(S))
     normed = torch.empty(rows, D, dtype=torch.bfloat16, device="cuda")
-    put("streams_step", lambda: ops.streams_step(x, upd, f32(S), w, 1e-6, normed), rows * D * (8 * S + 2 + 2))
+    in_w = f32(S)
+    put("streams_step", lambda: ops.streams_step(x, upd, in_w, w, 1e-6, normed), rows * D * (8 * S + 2 + 2))
     h = f32(rows, D)
     put("add_rmsnorm (one stream)", lambda: ops.add_rmsnorm(h, delta, w, 1e-6, normed), rows * D * (4 + 4 + 2 + 2))
     # between the q/k/v product and the attention: rotation, padding, cache write (the value goes in with both maps)

@@ -15,7 +15,7 @@
 #include "common.h"
 
 #define ST_THREADS 256
-#define ST_MAX_STREAMS 8
+#define ST_MAX_STREAMS 16
 #define ST_MAX_PER_THREAD 32  // rows of up to 8,192 elements
 
 struct StreamArgs {
@@ -231,9 +231,9 @@ extern "C" int fg_streams_step_rows(const StreamArgs* args, int n_rows, int act_
 #define GO(TA, TW)                                                                               \
   do {                                                                                           \
     if (a.dim % 4 == 0 && a.dim <= 1024 && S <= 4) VEC(TA, TW, 1, 4);                            \
-    else if (a.dim % 4 == 0 && a.dim <= 1024) VEC(TA, TW, 1, 8);                                 \
+    else if (a.dim % 4 == 0 && a.dim <= 1024 && S <= 8) VEC(TA, TW, 1, 8);                            \
     else if (a.dim % 4 == 0 && a.dim <= 2048 && S <= 4) VEC(TA, TW, 2, 4);                       \
-    else if (a.dim % 4 == 0 && a.dim <= 2048) VEC(TA, TW, 2, 8);                                 \
+    else if (a.dim % 4 == 0 && a.dim <= 2048 && S <= 8) VEC(TA, TW, 2, 8);                            \
     else if (a.dim % 4 == 0 && a.dim <= 4096 && S <= 4) VEC(TA, TW, 4, 4);                       \
     else if (a.dim <= 2 * ST_THREADS) streams_step_kernel<TA, TW, 2><<<n_rows, ST_THREADS, 0, stream>>>(a);  \
     else if (a.dim <= 8 * ST_THREADS) streams_step_kernel<TA, TW, 8><<<n_rows, ST_THREADS, 0, stream>>>(a);  \

@@ -1375,7 +1375,7 @@ class _StreamArgs(ctypes.Structure):
                 ("eps", ctypes.c_float)]
 
 
-STREAMS_MAX = 8
+STREAMS_MAX = 16
 
 
 def streams_spread(h: torch.Tensor, n_streams: int) -> torch.Tensor:

@@ -59,7 +59,7 @@ def _close_to_plain(got, want, noise, dtype, what, routed):
 
 # ------------------------------------------------------------------ kernels alone
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("S,T,D", [(1, 5, 40), (3, 7, 200), (4, 70, 1000), (8, 3, 2304), (5, 4, 1536), (2, 6, 42), (3, 5, 4096), (7, 9, 1024)])
+@pytest.mark.parametrize("S,T,D", [(1, 5, 40), (3, 7, 200), (4, 70, 1000), (8, 3, 2304), (5, 4, 1536), (2, 6, 42), (3, 5, 4096), (7, 9, 1024), (11, 3, 512), (16, 2, 100)])
 def test_streams_step_and_spread(dtype, S, T, D):
     from fastgen_amd.kernels import ops, twins
 
